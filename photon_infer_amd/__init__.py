@@ -1,0 +1,13 @@
+"""photon_infer_amd: a small, whole LLM inference engine for one AMD MI355X GPU."""
+from .errors import (CacheError, ConfigError, ErrorCode, KernelError, KernelLibraryMissing, OutOfPagesError,
+                     PhotonError, RequestError, UnsupportedModelError, WeightError)
+from .registry import (build_model_spec, get_architecture, load_config, register_architecture,
+                       registered_architectures)
+
+__version__ = "0.1.0"
+
+__all__ = [
+    "CacheError", "ConfigError", "ErrorCode", "KernelError", "KernelLibraryMissing", "OutOfPagesError",
+    "PhotonError", "RequestError", "UnsupportedModelError", "WeightError", "build_model_spec",
+    "get_architecture", "load_config", "register_architecture", "registered_architectures",
+]

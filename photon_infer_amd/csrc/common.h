@@ -1,0 +1,96 @@
+// Shared helpers of the gfx950 kernels: storage types, conversions, wave64 reductions,
+// and the error channel of the C entry points.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdarg.h>
+
+#define PI_WAVE 64
+
+// dtype tags shared with the Python binding
+enum PiDType : int { PI_F32 = 0, PI_BF16 = 1 };
+
+// bfloat16 is stored as its 16 bits; arithmetic is always float.
+struct bf16_t {
+  uint16_t bits;
+};
+
+__host__ __device__ inline float to_float(float v) { return v; }
+__host__ __device__ inline float to_float(bf16_t v) {
+  union { uint32_t u; float f; } c;
+  c.u = ((uint32_t)v.bits) << 16;
+  return c.f;
+}
+
+// round to nearest, ties to even; NaN stays NaN
+__host__ __device__ inline uint16_t f32_to_bf16_bits(float f) {
+  union { uint32_t u; float f; } c;
+  c.f = f;
+  uint32_t u = c.u;
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (uint16_t)(u >> 16);
+}
+
+template <typename T> __host__ __device__ inline T from_float(float v);
+template <> __host__ __device__ inline float from_float<float>(float v) { return v; }
+template <> __host__ __device__ inline bf16_t from_float<bf16_t>(float v) {
+  bf16_t r;
+  r.bits = f32_to_bf16_bits(v);
+  return r;
+}
+
+// ---- wave64 reductions (every lane gets the result)
+__device__ inline float wave_sum(float v) {
+#pragma unroll
+  for (int off = PI_WAVE / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, PI_WAVE);
+  return v;
+}
+__device__ inline float wave_max(float v) {
+#pragma unroll
+  for (int off = PI_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, PI_WAVE));
+  return v;
+}
+
+// Block-wide sum for blocks of up to 1024 threads (16 waves); `scratch` holds 16 floats.
+__device__ inline float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x / PI_WAVE, lane = threadIdx.x % PI_WAVE;
+  const int nwaves = (blockDim.x + PI_WAVE - 1) / PI_WAVE;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < nwaves; ++w) total += scratch[w];
+  return total;
+}
+
+// ---- error channel: entry points return 0 or a negative code and leave a message
+inline thread_local char pi_error_message[1024] = {0};
+
+// Each shared library defines its own accessor: PI_DEFINE_MODULE(core) gives
+// `const char* pi_core_last_error()`.
+#define PI_DEFINE_MODULE(name) \
+  extern "C" const char* pi_##name##_last_error() { return pi_error_message; }
+
+inline int pi_fail(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(pi_error_message, sizeof(pi_error_message), fmt, ap);
+  va_end(ap);
+  return -1;
+}
+
+inline int pi_check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return pi_fail("%s: launch failed: %s", what, hipGetErrorString(e));
+  return 0;
+}
+
+#define PI_REQUIRE(cond, ...) \
+  do {                        \
+    if (!(cond)) return pi_fail(__VA_ARGS__); \
+  } while (0)
+
+static inline int ceil_div(long a, long b) { return (int)((a + b - 1) / b); }

@@ -1,0 +1,196 @@
+// Embedding gather, RMS norm (optionally on gathered rows), SwiGLU, and the fused
+// position-rotation + paged key/value write.  All sizes are run-time values.
+#include "common.h"
+
+PI_DEFINE_MODULE(core)
+
+// ------------------------------------------------------------------ embedding
+// out[t, :] = float(table[ids[t], :]).  An id outside [0, V) fills the row with NaN:
+// loud in every later result, and no access outside the table.
+template <typename TW>
+__global__ void embedding_kernel(float* __restrict__ out, const TW* __restrict__ table,
+                                 const int* __restrict__ ids, int D, int V) {
+  const long t = blockIdx.x;
+  const int id = ids[t];
+  float* o = out + t * D;
+  if (id < 0 || id >= V) {
+    for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = __builtin_nanf("");
+    return;
+  }
+  const TW* row = table + (long)id * D;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = to_float(row[i]);
+}
+
+extern "C" int pi_embedding(float* out, const void* table, int table_dtype, const int* ids, int T, int D,
+                            int V, hipStream_t stream) {
+  PI_REQUIRE(T >= 0 && D > 0 && V > 0, "embedding: bad sizes T=%d D=%d V=%d", T, D, V);
+  if (T == 0) return 0;
+  const int threads = D >= 256 ? 256 : 64;
+  if (table_dtype == PI_F32)
+    hipLaunchKernelGGL(embedding_kernel<float>, dim3(T), dim3(threads), 0, stream, out, (const float*)table, ids, D, V);
+  else if (table_dtype == PI_BF16)
+    hipLaunchKernelGGL(embedding_kernel<bf16_t>, dim3(T), dim3(threads), 0, stream, out, (const bf16_t*)table, ids, D, V);
+  else
+    return pi_fail("embedding: unsupported table dtype %d", table_dtype);
+  return pi_check_launch("embedding");
+}
+
+// ------------------------------------------------------------------ RMS norm
+// y[m, :] = w * (x[r, :] * (1 / sqrt(mean(x[r, :]^2) + eps))), r = rows ? rows[m] : m.
+// Sum of squares, root and scaling in float32; one rounding on store.
+template <typename TO, typename TW>
+__global__ void rmsnorm_kernel(TO* __restrict__ out, const float* __restrict__ x, const int* __restrict__ rows,
+                               const TW* __restrict__ w, float eps, int D) {
+  __shared__ float scratch[16];
+  const long m = blockIdx.x;
+  const long r = rows ? rows[m] : m;
+  const float* xr = x + r * D;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) {
+    const float v = xr[i];
+    ss += v * v;
+  }
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+  TO* o = out + m * D;
+  for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = from_float<TO>(to_float(w[i]) * (xr[i] * inv));
+}
+
+extern "C" int pi_rmsnorm(void* out, int out_dtype, const float* x, const int* rows, const void* w, int w_dtype,
+                          float eps, int M, int D, hipStream_t stream) {
+  PI_REQUIRE(M >= 0 && D > 0, "rmsnorm: bad sizes M=%d D=%d", M, D);
+  if (M == 0) return 0;
+  const int threads = D >= 1024 ? 256 : (D >= 256 ? 128 : 64);
+#define LAUNCH(TO, TW) \
+  hipLaunchKernelGGL((rmsnorm_kernel<TO, TW>), dim3(M), dim3(threads), 0, stream, (TO*)out, x, rows, (const TW*)w, eps, D)
+  if (out_dtype == PI_F32 && w_dtype == PI_F32) LAUNCH(float, float);
+  else if (out_dtype == PI_F32 && w_dtype == PI_BF16) LAUNCH(float, bf16_t);
+  else if (out_dtype == PI_BF16 && w_dtype == PI_F32) LAUNCH(bf16_t, float);
+  else if (out_dtype == PI_BF16 && w_dtype == PI_BF16) LAUNCH(bf16_t, bf16_t);
+  else return pi_fail("rmsnorm: unsupported dtypes out=%d weight=%d", out_dtype, w_dtype);
+#undef LAUNCH
+  return pi_check_launch("rmsnorm");
+}
+
+// ------------------------------------------------------------------ SwiGLU
+// out[t, i] = g / (1 + exp(-g)) * u with g = gu[t, i], u = gu[t, I + i]; float32 math.
+template <typename T>
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, long total, int I) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= total) return;
+  const long t = idx / I;
+  const int i = (int)(idx - t * I);
+  const float g = to_float(gu[t * 2 * I + i]);
+  const float u = to_float(gu[t * 2 * I + I + i]);
+  out[idx] = from_float<T>(g / (1.0f + expf(-g)) * u);
+}
+
+extern "C" int pi_swiglu(void* out, const void* gu, int dtype, int T, int I, hipStream_t stream) {
+  PI_REQUIRE(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
+  if (T == 0) return 0;
+  const long total = (long)T * I;
+  const int threads = 256;
+  const long blocks = (total + threads - 1) / threads;
+  PI_REQUIRE(blocks < 2147483647L, "swiglu: too many elements (%ld)", total);
+  if (dtype == PI_F32)
+    hipLaunchKernelGGL(swiglu_kernel<float>, dim3((unsigned)blocks), dim3(threads), 0, stream, (float*)out, (const float*)gu, total, I);
+  else if (dtype == PI_BF16)
+    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3((unsigned)blocks), dim3(threads), 0, stream, (bf16_t*)out, (const bf16_t*)gu, total, I);
+  else
+    return pi_fail("swiglu: unsupported dtype %d", dtype);
+  return pi_check_launch("swiglu");
+}
+
+// ------------------------------------------------------------------ rotation + cache write
+// One wave per (token, head).  Heads 0..nh-1 are queries (rotated in place); then, when
+// the layer writes its cache, nkv key heads (rotated, stored to the page of the token's
+// position) and nkv value heads (stored as they are).
+// Cache layout: [page, kv_head, slot_in_page, head_dim].
+// angle = float(pos) * inv_freq[j]; pair j is (x[j], x[j + R/2]) or, interleaved,
+// (x[2j], x[2j+1]); (a, b) <- (a cos - b sin, a sin + b cos).  Dims >= R are copied.
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
+                                     const T* __restrict__ v, long v_stride, const int* __restrict__ positions,
+                                     const int* __restrict__ req_of_token, const float* __restrict__ inv_freq,
+                                     int rotary_dim, int interleaved, int nh, int nkv_write, int nkv, int hd,
+                                     T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                     const int* __restrict__ block_table, int table_width, int page_size,
+                                     long num_pages) {
+  const long t = blockIdx.x;
+  const int h = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int pos = positions[t];
+  const T* src;
+  T* dst;
+  bool rotate = rotary_dim > 0;
+  if (h < nh) {
+    dst = q + t * q_stride + (long)h * hd;
+    src = dst;
+  } else {
+    const int hh = h - nh;
+    const bool is_v = hh >= nkv_write;
+    const int g = is_v ? hh - nkv_write : hh;
+    const int r = req_of_token[t];
+    const int blk = pos / page_size;
+    if (blk >= table_width) return;
+    const long page = block_table[(long)r * table_width + blk];
+    if (page < 0 || page >= num_pages) return;  // the host checks tables; never write outside the pool
+    const long off = ((page * nkv + g) * page_size + (pos % page_size)) * hd;
+    if (is_v) {
+      src = v + t * v_stride + (long)g * hd;
+      dst = v_cache + off;
+      rotate = false;
+    } else {
+      src = k + t * k_stride + (long)g * hd;
+      dst = k_cache + off;
+    }
+  }
+  if (rotate) {
+    const int half = rotary_dim / 2;
+    for (int j = lane; j < half; j += PI_WAVE) {
+      const int i0 = interleaved ? 2 * j : j;
+      const int i1 = interleaved ? 2 * j + 1 : j + half;
+      const float a = to_float(src[i0]);
+      const float b = to_float(src[i1]);
+      const float angle = (float)pos * inv_freq[j];
+      float s, c;
+      sincosf(angle, &s, &c);
+      dst[i0] = from_float<T>(a * c - b * s);
+      dst[i1] = from_float<T>(a * s + b * c);
+    }
+    if (dst != src)
+      for (int i = rotary_dim + lane; i < hd; i += PI_WAVE) dst[i] = src[i];
+  } else if (dst != src) {
+    for (int i = lane; i < hd; i += PI_WAVE) dst[i] = src[i];
+  }
+}
+
+extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
+                                int dtype, const int* positions, const int* req_of_token, const float* inv_freq,
+                                int rotary_dim, int interleaved, int T, int nh, int nkv, int hd, int write_kv,
+                                void* k_cache, void* v_cache, const int* block_table, int table_width,
+                                int page_size, long num_pages, hipStream_t stream) {
+  PI_REQUIRE(T >= 0 && nh >= 0 && nkv >= 0 && hd > 0, "rope_kv_write: bad sizes T=%d heads=%d kv_heads=%d head_dim=%d", T, nh, nkv, hd);
+  PI_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && rotary_dim % 2 == 0, "rope_kv_write: rotary_dim %d must be even and <= head_dim %d", rotary_dim, hd);
+  PI_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "rope_kv_write: rotation asked for without a frequency table");
+  if (write_kv) {
+    PI_REQUIRE(k && v && k_cache && v_cache && block_table && req_of_token, "rope_kv_write: cache write asked for without k/v/cache/table");
+    PI_REQUIRE(page_size > 0 && table_width > 0 && num_pages > 0, "rope_kv_write: bad cache geometry page_size=%d table_width=%d pages=%ld", page_size, table_width, num_pages);
+  }
+  const int heads = nh + (write_kv ? 2 * nkv : 0);
+  if (T == 0 || heads == 0) return 0;
+  PI_REQUIRE(heads <= 65535, "rope_kv_write: too many heads (%d)", heads);
+  const dim3 grid(T, heads), block(PI_WAVE);
+  const int nkv_write = write_kv ? nkv : 0;
+  if (dtype == PI_F32)
+    hipLaunchKernelGGL(rope_kv_write_kernel<float>, grid, block, 0, stream, (float*)q, q_stride, (const float*)k, k_stride,
+                       (const float*)v, v_stride, positions, req_of_token, inv_freq, rotary_dim, interleaved, nh, nkv_write,
+                       nkv, hd, (float*)k_cache, (float*)v_cache, block_table, table_width, page_size, num_pages);
+  else if (dtype == PI_BF16)
+    hipLaunchKernelGGL(rope_kv_write_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)q, q_stride, (const bf16_t*)k, k_stride,
+                       (const bf16_t*)v, v_stride, positions, req_of_token, inv_freq, rotary_dim, interleaved, nh, nkv_write,
+                       nkv, hd, (bf16_t*)k_cache, (bf16_t*)v_cache, block_table, table_width, page_size, num_pages);
+  else
+    return pi_fail("rope_kv_write: unsupported dtype %d", dtype);
+  return pi_check_launch("rope_kv_write");
+}

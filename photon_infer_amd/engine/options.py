@@ -1,0 +1,46 @@
+"""Engine options: every constant the reference scatters through its sources
+(chunk 256 and max_sequences 32 in include/photon/scheduler/continuous_batch_engine.hpp:61-66,
+block size 16 and the pool size in demo/batched_infer_multi_prompts.cpp:355-358) as a field.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from ..errors import PhotonError
+
+_DTYPES = {
+    "bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
+    "float32": torch.float32, "fp32": torch.float32, "f32": torch.float32,
+}
+
+
+def parse_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name in (torch.bfloat16, torch.float32):
+            return name
+        raise PhotonError(f"compute dtype must be bfloat16 or float32, got {name}")
+    try:
+        return _DTYPES[str(name).lower()]
+    except KeyError:
+        raise PhotonError(f"compute dtype must be bfloat16 or float32, got '{name}'") from None
+
+
+@dataclass
+class EngineOptions:
+    dtype: object = "bfloat16"           # compute dtype: "bfloat16" or "float32"
+    block_size: int = 16                 # tokens per cache page
+    num_blocks: Optional[int] = None     # pages per cache group; None: from max_cache_tokens
+    max_cache_tokens: Optional[int] = None  # tokens the page pool holds; None: max_batch * max_model_len
+    max_batch: int = 32                  # most live requests (= state slots)
+    max_step_tokens: int = 2048          # token budget of one step
+    chunk_size: int = 256                # largest prompt portion of one request in one step
+    max_model_len: Optional[int] = None  # longest sequence; None: the model's max positions
+    seed: int = 0
+    device: str = "cuda:0"
+    use_graphs: bool = True              # replay HIP graphs for decode-only steps
+
+    def resolved_dtype(self) -> torch.dtype:
+        return parse_dtype(self.dtype)

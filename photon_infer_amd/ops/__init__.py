@@ -1,0 +1,261 @@
+"""Python face of the HIP kernels: shape / dtype / device checks, then one C call.
+
+Every function works on tensors that live on the GPU and launches on torch's current
+stream.  There is no CPU path: a tensor on the CPU, or a kernel library that cannot
+be built or loaded, is an error.
+
+Dispatch rule: bfloat16 operands whose sizes the matrix-core kernels take go to those
+kernels (module "bf16"); everything else - float32, mixed storage types, odd sizes -
+goes to the general kernels (module "core"), which take any size.
+``use_fast_kernels(False)`` forces the general kernels (tests compare the two).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from ..errors import KernelError
+from . import _lib
+
+PI_F32, PI_BF16 = 0, 1
+MAX_HEAD_DIM = 256
+
+_FAST = True
+
+
+def use_fast_kernels(enabled: bool) -> bool:
+    """Switch the matrix-core kernels on or off; returns the previous setting."""
+    global _FAST
+    prev, _FAST = _FAST, bool(enabled)
+    return prev
+
+
+def fast_kernels_enabled() -> bool:
+    return _FAST
+
+
+def ensure_loaded(dtype: torch.dtype) -> None:
+    """Build / load what a model of compute dtype ``dtype`` needs."""
+    _lib.load("core")
+    if dtype == torch.bfloat16 and _FAST and _lib.build.MODULES["bf16"]:
+        _lib.load("bf16")
+
+
+# ----------------------------------------------------------------------------- helpers
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return PI_F32
+    if t.dtype == torch.bfloat16:
+        return PI_BF16
+    raise KernelError(f"kernels take float32 or bfloat16 tensors, got {t.dtype}")
+
+
+def _gpu(*tensors: Optional[torch.Tensor]) -> None:
+    for t in tensors:
+        if t is not None and not t.is_cuda:
+            raise KernelError("kernels run on the GPU only; got a tensor on " + str(t.device))
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _rows(t: torch.Tensor, what: str) -> int:
+    """Row stride (elements) of a 2-D tensor whose rows are dense."""
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise KernelError(f"{what}: expected a 2-D tensor with dense rows, got shape {tuple(t.shape)} strides {t.stride()}")
+    return t.stride(0) if t.shape[0] > 1 else max(t.stride(0), t.shape[1])
+
+
+def _i32(t: torch.Tensor, what: str, n: Optional[int] = None) -> None:
+    if t.dtype != torch.int32 or not t.is_contiguous():
+        raise KernelError(f"{what}: expected a contiguous int32 tensor, got {t.dtype}")
+    if n is not None and t.numel() < n:
+        raise KernelError(f"{what}: expected at least {n} entries, got {t.numel()}")
+
+
+def check_attention_sizes(num_heads: int, num_kv_heads: int, head_dim: int) -> None:
+    """Sizes the attention kernels take; anything else is refused here, by name."""
+    if num_heads <= 0 or num_kv_heads <= 0 or num_heads % num_kv_heads:
+        raise KernelError(f"attention: {num_heads} heads is not a positive multiple of {num_kv_heads} kv heads")
+    if head_dim <= 0 or head_dim % 16 or head_dim > MAX_HEAD_DIM:
+        raise KernelError(f"attention: head_dim {head_dim} must be a multiple of 16 up to {MAX_HEAD_DIM}")
+
+
+# ----------------------------------------------------------------------------- ops
+def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None:
+    """out[t, :] = float32(table[ids[t], :])."""
+    _gpu(out, table, ids)
+    T, D = out.shape
+    if out.dtype != torch.float32 or not out.is_contiguous():
+        raise KernelError("embedding: output must be contiguous float32")
+    if table.dim() != 2 or table.shape[1] != D or not table.is_contiguous():
+        raise KernelError(f"embedding: table shape {tuple(table.shape)} does not match width {D}")
+    _i32(ids, "embedding ids", T)
+    _lib.call("core", "pi_embedding", out.data_ptr(), table.data_ptr(), _dt(table), ids.data_ptr(), T, D,
+              table.shape[0], _stream())
+
+
+def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float,
+            rows: Optional[torch.Tensor] = None) -> None:
+    """out[m, :] = weight * x[r, :] / sqrt(mean(x[r, :]^2) + eps), r = rows[m] (or m)."""
+    _gpu(out, x, weight, rows)
+    M, D = out.shape
+    if x.dtype != torch.float32 or not x.is_contiguous() or x.dim() != 2 or x.shape[1] != D:
+        raise KernelError(f"rmsnorm: input must be contiguous float32 [*, {D}], got {x.dtype} {tuple(x.shape)}")
+    if not out.is_contiguous() or weight.shape != (D,) or not weight.is_contiguous():
+        raise KernelError(f"rmsnorm: output must be contiguous and weight [{D}], got weight {tuple(weight.shape)}")
+    if rows is None:
+        if x.shape[0] != M:
+            raise KernelError(f"rmsnorm: {x.shape[0]} input rows for {M} output rows")
+    else:
+        _i32(rows, "rmsnorm rows", M)
+    _lib.call("core", "pi_rmsnorm", out.data_ptr(), _dt(out), x.data_ptr(), _ptr(rows), weight.data_ptr(),
+              _dt(weight), float(eps), M, D, _stream())
+
+
+def swiglu(out: torch.Tensor, gate_up: torch.Tensor) -> None:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
+    _gpu(out, gate_up)
+    T, I = out.shape
+    if gate_up.shape != (T, 2 * I) or gate_up.dtype != out.dtype or not (out.is_contiguous() and gate_up.is_contiguous()):
+        raise KernelError(f"swiglu: expected gate_up [{T}, {2 * I}] of {out.dtype}, got {tuple(gate_up.shape)} {gate_up.dtype}")
+    _lib.call("core", "pi_swiglu", out.data_ptr(), gate_up.data_ptr(), _dt(out), T, I, _stream())
+
+
+def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, accumulate: bool = False) -> None:
+    """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation."""
+    _gpu(out, a, w)
+    if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
+        raise KernelError("gemm: operands must be 2-D")
+    M, K = a.shape
+    N = w.shape[0]
+    if w.shape[1] != K or out.shape != (M, N):
+        raise KernelError(f"gemm: shapes do not agree: a {tuple(a.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)}")
+    if accumulate and out.dtype != torch.float32:
+        raise KernelError("gemm: accumulation needs a float32 output")
+    lda, ldw, ldc = _rows(a, "gemm a"), _rows(w, "gemm w"), _rows(out, "gemm out")
+    if M == 0:
+        return
+    if _FAST and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
+        from . import fast
+        if fast.gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc):
+            return
+    _lib.call("core", "pi_gemm_general", out.data_ptr(), _dt(out), ldc, a.data_ptr(), _dt(a), lda, w.data_ptr(),
+              _dt(w), ldw, M, N, K, int(accumulate), _stream())
+
+
+def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, hd: int, page_size: int, dtype) -> int:
+    if k_cache.shape != v_cache.shape or k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (nkv, page_size, hd):
+        raise KernelError(f"cache: expected [pages, {nkv}, {page_size}, {hd}], got {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
+    if k_cache.dtype != dtype or v_cache.dtype != dtype or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
+        raise KernelError(f"cache: must be contiguous {dtype}, got {k_cache.dtype}")
+    return k_cache.shape[0]
+
+
+def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], positions: torch.Tensor,
+                  req_of_token: torch.Tensor, rotary, num_heads: int, num_kv_heads: int, head_dim: int,
+                  k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
+                  block_table: Optional[torch.Tensor], page_size: int) -> None:
+    """Rotate q in place by each token's position; rotate k and store k, v into the pages.
+
+    ``rotary`` = (inv_freq float32 [R/2], R, interleaved) or None for no rotation.
+    ``k``/``v`` None: queries only (the layer reads a cache that another one writes).
+    """
+    _gpu(q, k, v, positions, req_of_token, k_cache, v_cache, block_table)
+    T = q.shape[0]
+    check_attention_sizes(num_heads, num_kv_heads, head_dim)
+    if q.shape[1] != num_heads * head_dim:
+        raise KernelError(f"rope: q has {q.shape[1]} columns, expected {num_heads * head_dim}")
+    _i32(positions, "positions", T)
+    write = k is not None
+    inv_freq, rdim, inter = (None, 0, False) if rotary is None else rotary
+    if inv_freq is not None and (inv_freq.dtype != torch.float32 or inv_freq.numel() != rdim // 2 or not inv_freq.is_contiguous()):
+        raise KernelError(f"rope: frequency table must be float32 [{rdim // 2}]")
+    if not write and rdim == 0:
+        return
+    pages = 0
+    if write:
+        if v is None or k.shape != (T, num_kv_heads * head_dim) or v.shape != k.shape or k.dtype != q.dtype or v.dtype != q.dtype:
+            raise KernelError(f"rope: k/v must be [{T}, {num_kv_heads * head_dim}] of {q.dtype}")
+        pages = _check_cache(k_cache, v_cache, num_kv_heads, head_dim, page_size, q.dtype)
+        _i32(req_of_token, "req_of_token", T)
+        if block_table.dim() != 2 or block_table.dtype != torch.int32 or not block_table.is_contiguous():
+            raise KernelError("rope: block table must be contiguous int32 [requests, width]")
+    _lib.call(
+        "core", "pi_rope_kv_write", q.data_ptr(), _rows(q, "q"), _ptr(k), _rows(k, "k") if write else 0, _ptr(v),
+        _rows(v, "v") if write else 0, _dt(q), positions.data_ptr(), _ptr(req_of_token) if write else None,
+        _ptr(inv_freq), rdim, int(bool(inter)), T, num_heads, num_kv_heads, head_dim, int(write),
+        _ptr(k_cache) if write else None, _ptr(v_cache) if write else None, _ptr(block_table) if write else None,
+        block_table.shape[1] if write else 0, page_size if write else 0, pages, _stream())
+
+
+def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                    block_table: torch.Tensor, ctx, num_heads: int, num_kv_heads: int, head_dim: int,
+                    page_size: int, scale: float, window: int = 0) -> None:
+    """Causal attention of every token of the step over its request's pages.
+
+    ``ctx`` carries ``positions`` and ``req_of_token`` ([T] int32) and, for the
+    matrix-core kernels, the work lists the step function made.
+    """
+    _gpu(out, q, k_cache, v_cache, block_table, ctx.positions, ctx.req_of_token)
+    T = q.shape[0]
+    check_attention_sizes(num_heads, num_kv_heads, head_dim)
+    if q.shape[1] != num_heads * head_dim or out.shape != (T, num_heads * head_dim) or out.dtype != q.dtype:
+        raise KernelError(f"attention: q {tuple(q.shape)} / out {tuple(out.shape)} do not match {num_heads} x {head_dim}")
+    pages = _check_cache(k_cache, v_cache, num_kv_heads, head_dim, page_size, q.dtype)
+    _i32(ctx.positions, "positions", T)
+    _i32(ctx.req_of_token, "req_of_token", T)
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or not block_table.is_contiguous():
+        raise KernelError("attention: block table must be contiguous int32 [requests, width]")
+    if T == 0:
+        return
+    if _FAST and q.dtype == torch.bfloat16:
+        from . import fast
+        if fast.paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
+                                page_size, scale, window, pages):
+            return
+    _lib.call("core", "pi_paged_attention_general", out.data_ptr(), _rows(out, "attention out"), q.data_ptr(),
+              _rows(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), _dt(q), block_table.data_ptr(),
+              block_table.shape[1], ctx.req_of_token.data_ptr(), ctx.positions.data_ptr(), T, num_heads,
+              num_kv_heads, head_dim, page_size, float(scale), int(window), pages, _stream())
+
+
+def sample(out: torch.Tensor, logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
+           uniform: Optional[torch.Tensor] = None) -> None:
+    """out[m] = argmax of row m (lowest index among equals) where temperature[m] <= 0 or
+    no temperatures are given; otherwise the first index whose cumulative
+    softmax(logits / temperature) reaches uniform[m]."""
+    _gpu(out, logits, temperature, uniform)
+    M, V = logits.shape
+    if logits.dtype != torch.float32:
+        raise KernelError("sample: logits must be float32")
+    _i32(out, "sample out", M)
+    for t, what in ((temperature, "temperature"), (uniform, "uniform")):
+        if t is not None and (t.dtype != torch.float32 or t.numel() < M or not t.is_contiguous()):
+            raise KernelError(f"sample: {what} must be contiguous float32 [{M}]")
+    if temperature is not None and uniform is None:
+        raise KernelError("sample: temperatures given without uniform numbers")
+    _lib.call("core", "pi_sample", out.data_ptr(), logits.data_ptr(), _rows(logits, "logits"), _ptr(temperature),
+              _ptr(uniform), M, V, _stream())
+
+
+# ----------------------------------------------------------------------------- work lists
+def plan_attention(q_lens, kv_lens, dtype) -> dict:
+    """Host-side work lists (int32 arrays to upload with the step's metadata) that the
+    matrix-core attention kernels want; empty for the general kernels."""
+    if _FAST and dtype == torch.bfloat16:
+        from . import fast
+        return fast.plan_attention(q_lens, kv_lens)
+    return {}
+
+
+def attach_attention_plan(ctx, plan: dict, views: dict) -> None:
+    if plan:
+        from . import fast
+        fast.attach_attention_plan(ctx, plan, views)

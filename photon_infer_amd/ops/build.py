@@ -1,0 +1,158 @@
+"""Builds the HIP kernel libraries for gfx950 with hipcc, in-tree.
+
+Sources live in ``photon_infer_amd/csrc``; each *module* is a handful of ``.hip`` files
+linked into ``csrc/_build/libphoton_<module>.so``.  A module is compiled when first
+needed (or when its sources changed since the library was built), one hipcc process per
+file in parallel, with a progress line every few seconds on stderr.
+"""
+from __future__ import annotations
+
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import threading
+import time
+from concurrent.futures import ThreadPoolExecutor
+from typing import Dict, List
+
+from ..errors import KernelLibraryMissing
+
+CSRC_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
+
+# module -> sources.  "core" holds every kernel the float32 path needs; "bf16" adds the
+# matrix-core kernels that only the bfloat16 path uses.
+MODULES: Dict[str, List[str]] = {
+    "core": ["elementwise.hip", "gemm_general.hip", "attention_general.hip", "sampling.hip"],
+    "bf16": [],
+}
+HEADERS = ["common.h", "mfma.h"]
+
+ARCH = "gfx950"
+HIPCC_FLAGS = [
+    f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    # packed float32 instructions off for device code (the host pass does not know the feature)
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-result",
+]
+
+
+def _log(msg: str) -> None:
+    print(f"[photon_infer_amd] {msg}", file=sys.stderr, flush=True)
+
+
+def _hipcc() -> str:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.isfile(cand):
+            return cand
+    raise KernelLibraryMissing("hipcc was not found (looked at $HIPCC, PATH and /opt/rocm/bin); "
+                               "the kernels cannot be built and there is no fallback")
+
+
+def _build_dir() -> str:
+    d = os.path.join(CSRC_DIR, "_build")
+    try:
+        os.makedirs(d, exist_ok=True)
+        probe = os.path.join(d, f".w{os.getpid()}")
+        with open(probe, "w"):
+            pass
+        os.remove(probe)
+        return d
+    except OSError:
+        d = os.path.join(tempfile.gettempdir(), f"photon_infer_amd_build_{os.getuid()}")
+        os.makedirs(d, exist_ok=True)
+        return d
+
+
+def source_hash(module: str) -> str:
+    h = hashlib.sha256(" ".join(HIPCC_FLAGS).encode())
+    for name in MODULES[module] + HEADERS:
+        path = os.path.join(CSRC_DIR, name)
+        if os.path.isfile(path):
+            with open(path, "rb") as f:
+                h.update(name.encode() + b"\0" + f.read())
+    return h.hexdigest()
+
+
+def library_path(module: str) -> str:
+    return os.path.join(_build_dir(), f"libphoton_{module}.so")
+
+
+def is_current(module: str) -> bool:
+    lib = library_path(module)
+    stamp = lib + ".hash"
+    if not (os.path.isfile(lib) and os.path.isfile(stamp)):
+        return False
+    with open(stamp) as f:
+        return f.read().strip() == source_hash(module)
+
+
+def _run(cmd: List[str], what: str) -> None:
+    env = dict(os.environ)
+    env.setdefault("HOME", tempfile.gettempdir())  # hipcc wants a HOME for its caches
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, env=env)
+    if proc.returncode != 0:
+        raise KernelLibraryMissing(f"building {what} failed (exit {proc.returncode}):\n{' '.join(cmd)}\n{proc.stdout}")
+    noise = "is not a recognized feature for this target"
+    out = "\n".join(l for l in proc.stdout.splitlines() if noise not in l).strip()
+    if out:
+        _log(f"{what}: compiler output:\n{out}")
+
+
+def build_module(module: str, force: bool = False, quiet: bool = False) -> str:
+    """Compile and link one module if it is missing or stale; returns the library path."""
+    if module not in MODULES:
+        raise KernelLibraryMissing(f"unknown kernel module '{module}'")
+    lib = library_path(module)
+    if not force and is_current(module):
+        return lib
+    hipcc = _hipcc()
+    bdir = _build_dir()
+    sources = MODULES[module]
+    missing = [s for s in sources if not os.path.isfile(os.path.join(CSRC_DIR, s))]
+    if missing:
+        raise KernelLibraryMissing(f"kernel sources missing for module '{module}': {missing}")
+    t0 = time.time()
+    if not quiet:
+        _log(f"building kernel module '{module}' for {ARCH} ({len(sources)} files) ...")
+    done = threading.Event()
+
+    def heartbeat():
+        while not done.wait(10.0):
+            _log(f"  still compiling '{module}' ({time.time() - t0:.0f} s)")
+
+    hb = threading.Thread(target=heartbeat, daemon=True)
+    if not quiet:
+        hb.start()
+    objs = []
+    try:
+        def compile_one(src: str) -> str:
+            obj = os.path.join(bdir, f"{module}_{os.path.splitext(src)[0]}.{os.getpid()}.o")
+            _run([hipcc, *HIPCC_FLAGS, "-I", CSRC_DIR, "-c", os.path.join(CSRC_DIR, src), "-o", obj], src)
+            if not quiet:
+                _log(f"  compiled {src} ({time.time() - t0:.0f} s)")
+            return obj
+
+        with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
+            objs = list(pool.map(compile_one, sources))
+        tmp = f"{lib}.{os.getpid()}.tmp"
+        _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", tmp], f"libphoton_{module}.so")
+        os.replace(tmp, lib)
+        with open(lib + ".hash", "w") as f:
+            f.write(source_hash(module))
+    finally:
+        done.set()
+        for o in objs:
+            try:
+                os.remove(o)
+            except OSError:
+                pass
+    if not quiet:
+        _log(f"built {lib} in {time.time() - t0:.0f} s")
+    return lib
+
+
+def build_all(force: bool = True) -> List[str]:
+    return [build_module(m, force=force) for m in MODULES]

@@ -1,0 +1,189 @@
+"""Interfaces of the parts a layer is put together from, and their registries.
+
+A model is data: a list of blocks, each naming a norm, a mixer, a feed-forward and an
+arrangement, plus a run order.  Every part takes its sizes and constants as
+constructor parameters, declares the tensors it expects (relative names) and what it
+needs from the cache manager; none of them knows which model it sits in.
+
+The reference wires one fixed block (src/arch/transformer_block.cpp:28-58: two norms,
+seven matmuls, rope, mha, add, swiglu) and has no such seam; the interfaces below are
+what replaces it.
+
+Data flow convention: the residual stream ``x`` is float32 ``[T, hidden]`` in both
+compute modes.  A norm reads ``x`` and writes activations ``h`` in the compute dtype;
+a mixer or feed-forward reads ``h`` and *adds* its result into ``x``.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Any, Callable, Dict, List, Optional, Sequence
+
+import torch
+
+from ..errors import UnsupportedModelError
+from ..weights.loader import TensorSpec
+
+
+# --------------------------------------------------------------------------- cache needs
+@dataclass(frozen=True)
+class KVCacheSpec:
+    """Keys and values kept per token, in pages.
+
+    ``window`` = None keeps all keys; an integer W keeps the last W positions, so the
+    cache manager may hand back pages that the window has passed.
+    """
+
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """State of fixed size per request (shape without the slot dimension)."""
+
+    shape: tuple
+    dtype: torch.dtype = torch.float32
+
+
+# --------------------------------------------------------------------------- step context
+@dataclass
+class StepContext:
+    """What one step's kernels need to know about the batch; built by the step function.
+
+    Device tensors are int32.  ``T`` tokens belong to ``R`` requests; request r owns
+    tokens ``q_start[r] .. q_start[r+1]``, at absolute positions
+    ``kv_len[r] - q_len[r] ..  kv_len[r] - 1``.
+    """
+
+    T: int
+    R: int
+    dtype: torch.dtype                    # compute / activation dtype
+    token_ids: torch.Tensor               # [T]
+    positions: torch.Tensor               # [T] absolute position of each token
+    req_of_token: torch.Tensor            # [T] row of the token's request in this step
+    q_start: torch.Tensor                 # [R+1]
+    kv_len: torch.Tensor                  # [R] keys visible after this step's writes
+    slots: torch.Tensor                   # [R] per-request state slot
+    block_tables: Dict[int, torch.Tensor]  # cache group -> [R, width] page ids (-1 = none)
+    logit_rows: torch.Tensor              # [M] token rows whose logits are wanted
+    # host-side copies for launch planning (never read by kernels)
+    q_lens: Sequence[int] = ()
+    kv_lens: Sequence[int] = ()
+    max_q_len: int = 0
+    max_kv_len: int = 0
+    all_decode: bool = False
+    # attention work lists (device) made by the step function
+    decode_reqs: Optional[torch.Tensor] = None   # [Rd] requests with one token
+    num_decode: int = 0
+    tile_req: Optional[torch.Tensor] = None      # [NT] request of each query tile
+    tile_q0: Optional[torch.Tensor] = None       # [NT] first token (within the request's portion)
+    num_tiles: int = 0
+    tile_rows: int = 0
+    decode_splits: int = 1                       # key ranges per request in split-K decode
+    workspace: Any = None                        # engine-owned scratch tensors
+    host_slots: Sequence[int] = ()
+
+
+@dataclass
+class LayerCache:
+    """The view of the cache manager that one entry of the run order gets."""
+
+    group: int = -1                       # cache group of the pages (-1: no pages)
+    k: Optional[torch.Tensor] = None      # [pages, kv_heads, page_size, head_dim]
+    v: Optional[torch.Tensor] = None
+    page_size: int = 0
+    writes: bool = True                   # False: reads another entry's cache
+    state: Optional[torch.Tensor] = None  # [max_slots, *StateSpec.shape]
+
+
+# --------------------------------------------------------------------------- part bases
+class Part:
+    """Common behaviour: declare tensors, receive them, know the compute dtype."""
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return []
+
+    def load(self, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device: torch.device) -> None:
+        """Receive this part's tensors (relative names), already on ``device``."""
+        self.dtype = dtype
+        self.device = device
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """``x`` float32 [N, D] -> normalised rows in the compute dtype ([M, D] when
+        ``rows`` (int32 [M]) selects rows of ``x``)."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Encodes positions into queries and keys.
+
+    ``rotary_params()`` lets the attention mixer fuse the rotation into its cache-write
+    kernel; a scheme that is not a rotation returns None and implements ``apply``.
+    """
+
+    def rotary_params(self):
+        return None
+
+    def apply(self, q: torch.Tensor, k: torch.Tensor, ctx: StepContext) -> None:
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self):
+        """KVCacheSpec, StateSpec or None."""
+        return None
+
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
+        """Read activations ``h`` [T, D]; add the mixer's output into ``x`` (float32)."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
+        """Read activations ``h`` [T, D]; add the result into ``x`` (float32)."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    """An arrangement of norm(s), mixer and feed-forward around the residual stream."""
+
+    mixer: Mixer
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
+        raise NotImplementedError
+
+
+# --------------------------------------------------------------------------- registries
+class PartRegistry:
+    def __init__(self, what: str):
+        self.what = what
+        self._makers: Dict[str, Callable[..., Any]] = {}
+
+    def register(self, kind: str, maker: Callable[..., Any] | None = None):
+        """``register("name", cls)`` or ``@register("name")``."""
+        if maker is None:
+            def deco(m):
+                self._makers[kind] = m
+                return m
+            return deco
+        self._makers[kind] = maker
+        return maker
+
+    def make(self, kind: str, **params) -> Any:
+        if kind not in self._makers:
+            known = ", ".join(sorted(self._makers)) or "<none>"
+            raise UnsupportedModelError(f"{self.what} '{kind}' is not registered (registered: {known})")
+        return self._makers[kind](**params)
+
+    def kinds(self) -> tuple:
+        return tuple(sorted(self._makers))
+
+
+NORMS = PartRegistry("norm")
+MIXERS = PartRegistry("mixer")
+FEED_FORWARDS = PartRegistry("feed-forward")
+POSITION_ENCODINGS = PartRegistry("position encoding")
+BLOCKS = PartRegistry("block arrangement")

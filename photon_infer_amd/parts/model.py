@@ -1,0 +1,138 @@
+"""A decoder model as data: embedding, a list of blocks, a run order, final norm, head.
+
+Reference: src/arch/llama_model.cpp:30-46 builds embedding + N identical blocks +
+final norm + classifier and runs them in index order (:242-246, :583-593).  Here the
+run order is a list of entries; an entry names the block whose weights it runs and,
+optionally, an earlier entry whose cache it reads instead of writing one of its own.
+A block may appear in several entries.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import torch
+
+from ..errors import ConfigError
+from ..weights.loader import TensorSpec
+from .base import Block, KVCacheSpec, LayerCache, Norm, StateSpec, StepContext
+from .embedding import LMHead, TokenEmbedding
+
+
+@dataclass(frozen=True)
+class RunEntry:
+    layer: int                       # index into ModelSpec.layers
+    cache_of: Optional[int] = None   # index of an earlier RunEntry whose cache is read
+
+
+@dataclass
+class ModelSpec:
+    hidden_size: int
+    vocab_size: int
+    max_positions: int
+    embedding: Tuple[str, TokenEmbedding]
+    layers: List[Tuple[str, Block]]
+    final_norm: Tuple[str, Norm]
+    head: Tuple[str, LMHead]
+    run_order: List[RunEntry] = field(default_factory=list)
+    ignorable: Tuple[str, ...] = ()   # name patterns a folder may hold beyond the expected ones
+    eos_token_ids: Tuple[int, ...] = ()
+    bos_token_id: Optional[int] = None
+
+    def __post_init__(self):
+        if not self.run_order:
+            self.run_order = [RunEntry(i) for i in range(len(self.layers))]
+        for i, e in enumerate(self.run_order):
+            if not 0 <= e.layer < len(self.layers):
+                raise ConfigError(f"run order entry {i} names layer {e.layer} of {len(self.layers)}")
+            if e.cache_of is not None:
+                if not 0 <= e.cache_of < i:
+                    raise ConfigError(f"run order entry {i} reads the cache of entry {e.cache_of}, which is not earlier")
+                if self.run_order[e.cache_of].cache_of is not None:
+                    raise ConfigError(f"run order entry {i} reads the cache of entry {e.cache_of}, which owns none")
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = [s.with_prefix(self.embedding[0]) for s in self.embedding[1].tensor_specs()]
+        for prefix, block in self.layers:
+            specs += [s.with_prefix(prefix) for s in block.tensor_specs()]
+        specs += [s.with_prefix(self.final_norm[0]) for s in self.final_norm[1].tensor_specs()]
+        specs += [s.with_prefix(self.head[0]) for s in self.head[1].tensor_specs()]
+        return specs
+
+
+# ------------------------------------------------------------------ what the cache must hold
+@dataclass(frozen=True)
+class CacheGroupPlan:
+    """Run-order entries whose keys/values live in pages of one pool."""
+
+    window: Optional[int]
+    entries: Tuple[int, ...]             # run-order indices that own K/V pages
+    kv_shapes: Tuple[Tuple[int, int], ...]  # (kv_heads, head_dim) per entry
+
+
+@dataclass(frozen=True)
+class CachePlan:
+    groups: Tuple[CacheGroupPlan, ...]
+    states: Tuple[Tuple[int, StateSpec], ...]   # (run-order index, spec)
+    group_of_entry: Dict[int, int]
+
+
+def plan_cache(spec: ModelSpec) -> CachePlan:
+    """Group the run order's cache needs: one page pool per distinct window."""
+    by_window: Dict[Optional[int], List[Tuple[int, KVCacheSpec]]] = {}
+    states: List[Tuple[int, StateSpec]] = []
+    for i, e in enumerate(spec.run_order):
+        if e.cache_of is not None:
+            continue
+        need = spec.layers[e.layer][1].mixer.cache_spec()
+        if isinstance(need, KVCacheSpec):
+            by_window.setdefault(need.window, []).append((i, need))
+        elif isinstance(need, StateSpec):
+            states.append((i, need))
+        elif need is not None:
+            raise ConfigError(f"mixer of layer {e.layer} returned an unknown cache spec {need!r}")
+    groups, group_of_entry = [], {}
+    for g, (window, items) in enumerate(sorted(by_window.items(), key=lambda kv: (kv[0] is not None, kv[0] or 0))):
+        groups.append(CacheGroupPlan(window, tuple(i for i, _ in items),
+                                     tuple((n.num_kv_heads, n.head_dim) for _, n in items)))
+        for i, _ in items:
+            group_of_entry[i] = g
+    for i, e in enumerate(spec.run_order):
+        if e.cache_of is not None and e.cache_of in group_of_entry:
+            group_of_entry[i] = group_of_entry[e.cache_of]
+    return CachePlan(tuple(groups), tuple(states), group_of_entry)
+
+
+# ------------------------------------------------------------------ the runnable model
+class DecoderModel:
+    def __init__(self, spec: ModelSpec):
+        self.spec = spec
+        self.embedding = spec.embedding[1]
+        self.blocks = [b for _, b in spec.layers]
+        self.final_norm = spec.final_norm[1]
+        self.head = spec.head[1]
+        self.dtype: Optional[torch.dtype] = None
+
+    def load(self, tensors: Dict[str, torch.Tensor], dtype: torch.dtype, device) -> None:
+        """Hand each part its tensors (names relative to the part's prefix)."""
+        device = torch.device(device)
+        self.dtype, self.device = dtype, device
+
+        def sub(prefix: str) -> Dict[str, torch.Tensor]:
+            return {n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}
+
+        self.embedding.load(sub(self.spec.embedding[0]), dtype, device)
+        for prefix, block in self.spec.layers:
+            block.load(sub(prefix), dtype, device)
+        self.final_norm.load(sub(self.spec.final_norm[0]), dtype, device)
+        self.head.load(sub(self.spec.head[0]), dtype, device, tied_weight=self.embedding.weight)
+
+    def forward(self, ctx: StepContext, caches: Sequence[LayerCache]) -> Optional[torch.Tensor]:
+        """Run the step's tokens through the run order; float32 logits [M, vocab] at
+        ``ctx.logit_rows`` (None when no row is wanted)."""
+        x = self.embedding.forward(ctx.token_ids)
+        for i, entry in enumerate(self.spec.run_order):
+            self.blocks[entry.layer].forward(x, ctx, caches[i])
+        if ctx.logit_rows.shape[0] == 0:
+            return None
+        return self.head.forward(self.final_norm.forward(x, rows=ctx.logit_rows))

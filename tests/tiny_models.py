@@ -1,0 +1,52 @@
+"""Tiny Llama configurations for tests; they differ in every size and option."""
+from __future__ import annotations
+
+import os
+
+import torch
+
+from photon_infer_amd.config import LlamaConfig
+from photon_infer_amd.weights import write_random_model
+
+TINY_A = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=64, intermediate_size=176, num_hidden_layers=2,
+    num_attention_heads=4, num_key_value_heads=2, vocab_size=256, max_position_embeddings=128,
+    rms_norm_eps=1e-5, rope_theta=10000.0, rope_scaling=None, tie_word_embeddings=True,
+)
+TINY_A_INIT = dict(std=0.02, norm_init="ones", block_size=4)
+
+TINY_B = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=128, intermediate_size=320, num_hidden_layers=3,
+    num_attention_heads=4, num_key_value_heads=1, head_dim=32, vocab_size=384, max_position_embeddings=256,
+    rms_norm_eps=1e-6, rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=64),
+    tie_word_embeddings=False,
+)
+TINY_B_INIT = dict(std=0.05, norm_init="uniform", block_size=8)
+
+# head_dim * heads != hidden, 3 heads in 3 groups, widths that are no power of two, a
+# vocabulary that is no multiple of anything, linear frequency scaling, bigger weights so
+# attention is far from uniform
+TINY_C = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=96, intermediate_size=200, num_hidden_layers=4,
+    num_attention_heads=6, num_key_value_heads=3, head_dim=48, vocab_size=1001, max_position_embeddings=512,
+    rms_norm_eps=3e-5, rope_theta=1000.0, rope_scaling=dict(rope_type="linear", factor=2.0),
+    tie_word_embeddings=False,
+)
+TINY_C_INIT = dict(std=0.12, norm_init="uniform", block_size=16)
+
+ALL = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT)}
+
+
+def make_model_dir(tmp_path, name: str, seed: int = 0, storage: str = "bfloat16") -> str:
+    raw, init = ALL[name]
+    cfg = LlamaConfig.from_dict(raw)
+    d = os.path.join(str(tmp_path), f"tiny_{name}_{seed}_{storage}")
+    write_random_model(cfg, d, seed=seed, std=init["std"], norm_init=init["norm_init"], dtype=storage)
+    return d
+
+
+def random_tokens(n: int, vocab: int, seed: int):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randint(0, vocab, (n,), generator=g).tolist()
