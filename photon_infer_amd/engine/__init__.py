@@ -1,4 +1,7 @@
+from .engine import ContinuousBatchEngine, Engine
 from .options import EngineOptions, parse_dtype
+from .scheduler import ContinuousBatchScheduler, InferenceRequest, RequestState, ScheduledBatch
 from .step import ModelRunner, StepEntry
 
-__all__ = ["EngineOptions", "parse_dtype", "ModelRunner", "StepEntry"]
+__all__ = ["ContinuousBatchEngine", "Engine", "EngineOptions", "parse_dtype", "ContinuousBatchScheduler",
+           "InferenceRequest", "RequestState", "ScheduledBatch", "ModelRunner", "StepEntry"]

@@ -1,0 +1,123 @@
+"""The engine: requests in, tokens out, by continuous batching over ``ModelRunner.step``.
+
+Reference: ``ContinuousBatchEngine`` (include/photon/scheduler/continuous_batch_engine.hpp:48-315):
+``add_request`` -> ``run_until_complete`` (loop: ``schedule_next_batch`` ->
+``execute_batch_step``) -> ``get_result``.  The same names and meanings are kept; requests
+are given as token ids (text goes through the tokenizer of the command line).
+"""
+from __future__ import annotations
+
+import sys
+from typing import Dict, List, Optional, Sequence
+
+from ..errors import RequestError
+from ..sampling import Sampler, SamplingParams, uniform_draw
+from .options import EngineOptions
+from .scheduler import ContinuousBatchScheduler, InferenceRequest, ScheduledBatch, SchedulerStats
+from .step import ModelRunner, StepEntry
+
+
+class ContinuousBatchEngine:
+    def __init__(self, model_dir: str, options: Optional[EngineOptions] = None, **option_fields):
+        """``ContinuousBatchEngine(model_dir, dtype="bfloat16", max_batch=64, ...)``: any field
+        of EngineOptions may be given by keyword."""
+        if options is None:
+            options = EngineOptions(**option_fields)
+        elif option_fields:
+            raise RequestError("give either an EngineOptions object or option fields, not both")
+        self.options = options
+        self.runner = ModelRunner(model_dir, options)
+        self.scheduler = ContinuousBatchScheduler(
+            self.runner.cache, options.max_batch, options.max_step_tokens, options.chunk_size,
+            self.runner.max_model_len, owner=self.runner)
+        self.sampler = Sampler(self.runner.device)
+        self.eos_token_ids = tuple(self.runner.spec.eos_token_ids)
+        self.steps = 0
+
+    @property
+    def config(self):
+        return self.runner.config
+
+    # ------------------------------------------------------------------ requests
+    def add_request(self, prompt_tokens: Sequence[int], max_new_tokens: int = 128, temperature: float = 0.0,
+                    seed: Optional[int] = None, ignore_eos: bool = False, prompt: str = "") -> int:
+        vocab = self.runner.spec.vocab_size
+        for t in prompt_tokens:
+            if not 0 <= int(t) < vocab:
+                raise RequestError(f"token id {t} is outside the vocabulary of {vocab}")
+        params = SamplingParams(temperature=float(temperature), max_new_tokens=int(max_new_tokens),
+                                seed=-1 if seed is None else int(seed), ignore_eos=ignore_eos)
+        rid = self.scheduler.add_request(prompt_tokens, params, prompt)
+        if seed is None:  # a stream of its own, fixed by the engine's seed and the request's number
+            params.seed = (self.options.seed * 1_000_003 + rid) & 0x7FFFFFFFFFFFFFFF
+        return rid
+
+    def get_request(self, request_id: int) -> Optional[InferenceRequest]:
+        return self.scheduler.get_request(request_id)
+
+    def get_result(self, request_id: int) -> List[int]:
+        """Generated token ids of a finished request (empty while it is unfinished)."""
+        req = self.scheduler.get_request(request_id)
+        if req is None or not req.is_finished():
+            return []
+        return list(req.generated_tokens)
+
+    def get_stats(self) -> SchedulerStats:
+        return self.scheduler.get_stats()
+
+    # ------------------------------------------------------------------ running
+    def step(self) -> List[InferenceRequest]:
+        """Schedule and run one batch; returns the requests that finished in it."""
+        batch = self.scheduler.schedule_next_batch()
+        finished = list(batch.finished)
+        if batch.empty():
+            return finished
+        finished += self.execute_batch_step(batch)
+        return finished
+
+    def execute_batch_step(self, batch: ScheduledBatch) -> List[InferenceRequest]:
+        entries, sampled_reqs = [], []
+        for req, n in batch.items:
+            ends = req.num_computed_tokens + n == req.total_tokens()
+            entries.append(StepEntry(req.request_id, req.next_tokens(n), [n - 1] if ends else []))
+            if ends:
+                sampled_reqs.append(req)
+        logits = self.runner.step(entries)
+        tokens: List[int] = []
+        if sampled_reqs:
+            temps = [r.params.temperature for r in sampled_reqs]
+            draws = [uniform_draw(r.params.seed, r.num_generated()) if r.params.temperature > 0 else 0.0
+                     for r in sampled_reqs]
+            tokens = self.sampler.sample(logits, temps, draws)
+        done = []
+        for req, n in batch.items:
+            req.add_computed_tokens(n)
+        for req, tok in zip(sampled_reqs, tokens):
+            if not req.add_token(tok, self.eos_token_ids, self.runner.max_model_len):
+                done.append(req)
+        self.scheduler.update_after_step(done)
+        self.steps += 1
+        return done
+
+    def run_until_complete(self, print_progress: bool = False) -> None:
+        while self.scheduler.has_work():
+            if print_progress and self.steps % 10 == 0:
+                s = self.scheduler.get_stats()
+                print(f"Step {self.steps}: Running={s.num_running} Waiting={s.num_waiting} Finished={s.num_finished}",
+                      file=sys.stderr, flush=True)
+            self.step()
+        if print_progress:
+            s = self.scheduler.get_stats()
+            print(f"Complete! Total steps: {self.steps} Total requests: {s.total_requests}", file=sys.stderr, flush=True)
+
+    # ------------------------------------------------------------------ convenience
+    def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 128, temperature: float = 0.0,
+                 seed: Optional[int] = None, ignore_eos: bool = False) -> List[List[int]]:
+        """Generate for every prompt (token id lists); returns the new token ids of each."""
+        ids = [self.add_request(p, max_new_tokens, temperature,
+                                None if seed is None else seed + i, ignore_eos) for i, p in enumerate(prompts)]
+        self.run_until_complete()
+        return [self.get_result(i) for i in ids]
+
+
+Engine = ContinuousBatchEngine
