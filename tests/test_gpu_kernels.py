@@ -1,0 +1,329 @@
+"""Each kernel alone against its plain reference, at sizes other than the engine's."""
+import math
+
+import pytest
+import torch
+
+import plain_llama as P
+from gpu_tools import DEV, PagedKV, attention_ctx
+
+pytestmark = pytest.mark.gpu
+
+F32, BF16 = torch.float32, torch.bfloat16
+
+
+@pytest.fixture(autouse=True)
+def _ops():
+    from photon_infer_amd import ops
+    prev = ops.use_fast_kernels(True)
+    yield ops
+    ops.use_fast_kernels(prev)
+
+
+def gen(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def close(got, want, rel, what=""):
+    scale = max(1e-6, want.abs().max().item())
+    err = (got.float().cpu() - want.float()).abs().max().item()
+    assert err <= rel * scale, f"{what}: max error {err:.3e} exceeds {rel:.1e} x scale {scale:.3e}"
+
+
+# ------------------------------------------------------------------ embedding
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_embedding(_ops, dtype):
+    table = torch.randn(1001, 72, generator=gen(0)).to(dtype)
+    ids = torch.tensor([0, 1000, 5, 5, 77], dtype=torch.int32)
+    out = torch.empty(5, 72, dtype=F32, device=DEV)
+    _ops.embedding(out, table.to(DEV), ids.to(DEV))
+    assert torch.equal(out.cpu(), P.embedding(table.float(), ids.tolist()))
+    bad = torch.tensor([3, 1001, -1], dtype=torch.int32, device=DEV)   # outside the table: NaN rows, no fault
+    out = torch.zeros(3, 72, dtype=F32, device=DEV)
+    _ops.embedding(out, table.to(DEV), bad)
+    assert not out[0].isnan().any() and out[1:].isnan().all()
+
+
+# ------------------------------------------------------------------ RMS norm
+@pytest.mark.parametrize("D", [24, 100, 1000, 2048, 4100])
+@pytest.mark.parametrize("out_dtype,w_dtype", [(F32, F32), (BF16, BF16), (BF16, F32)])
+def test_rmsnorm(_ops, D, out_dtype, w_dtype):
+    x = torch.randn(7, D, generator=gen(D)) * 3 + 0.5
+    w = (torch.rand(D, generator=gen(1)) + 0.5).to(w_dtype)
+    out = torch.empty(7, D, dtype=out_dtype, device=DEV)
+    _ops.rmsnorm(out, x.to(DEV), w.to(DEV), 1e-6)
+    want = P.rmsnorm(x, w.float(), 1e-6)
+    close(out, want, 2e-6 if out_dtype == F32 else 2 ** -8, f"rmsnorm D={D}")
+    rows = torch.tensor([6, 0, 3], dtype=torch.int32, device=DEV)
+    out2 = torch.empty(3, D, dtype=out_dtype, device=DEV)
+    _ops.rmsnorm(out2, x.to(DEV), w.to(DEV), 1e-6, rows)
+    assert torch.equal(out2, out[[6, 0, 3]])
+
+
+def test_rmsnorm_reference_vectors(_ops):
+    # tests/ops/test_rmsnorm.cpp:102-181
+    x = torch.tensor([[1.0, 2.0, 3.0, 4.0], [2.0, 4.0, 6.0, 8.0]], device=DEV)
+    out = torch.empty(2, 4, device=DEV)
+    _ops.rmsnorm(out, x, torch.tensor([0.5, 1.0, 1.5, 2.0], device=DEV), 1e-5)
+    w = torch.tensor([0.5, 1.0, 1.5, 2.0])
+    assert torch.allclose(out[0].cpu(), w * x[0].cpu() / math.sqrt(7.5 + 1e-5), atol=1e-6)
+    assert torch.allclose(out[1].cpu(), w * x[1].cpu() / math.sqrt(30 + 1e-5), atol=1e-6)
+
+
+# ------------------------------------------------------------------ SwiGLU
+@pytest.mark.parametrize("dtype", [F32, BF16])
+def test_swiglu(_ops, dtype):
+    T, I = 5, 176
+    gu = (torch.randn(T, 2 * I, generator=gen(2)) * 4).to(dtype)
+    gu[0, :4] = torch.tensor([1.0, 2.0, 3.0, 4.0]).to(dtype)          # tests/ops/test_swiglu.cpp:159-216
+    gu[0, I:I + 4] = torch.tensor([0.5, 1.0, 1.5, 2.0]).to(dtype)
+    gu[1, :3] = torch.tensor([90.0, -90.0, 0.0]).to(dtype)
+    out = torch.empty(T, I, dtype=dtype, device=DEV)
+    _ops.swiglu(out, gu.to(DEV))
+    want = P.swiglu(gu[:, :I].float(), gu[:, I:].float())
+    close(out, want, 1e-6 if dtype == F32 else 2 ** -8, "swiglu")
+    assert not out.isnan().any() and out[1, 1].item() == 0 and out[1, 2].item() == 0
+
+
+# ------------------------------------------------------------------ matrix products
+GEMM_SHAPES = [(1, 14, 3), (2, 2, 3), (5, 176, 64), (33, 100, 72), (64, 384, 128), (70, 1001, 96), (1, 256, 64),
+               (130, 64, 200), (257, 320, 136), (8, 2048, 512), (300, 520, 264)]
+
+
+@pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
+@pytest.mark.parametrize("a_dtype,w_dtype,c_dtype", [(F32, F32, F32), (BF16, BF16, BF16), (BF16, BF16, F32), (BF16, F32, BF16)])
+@pytest.mark.parametrize("fast", [False, True])
+def test_gemm(_ops, M, N, K, a_dtype, w_dtype, c_dtype, fast):
+    if fast and not (a_dtype == BF16 and w_dtype == BF16):
+        pytest.skip("the matrix-core kernels take bfloat16 operands only")
+    _ops.use_fast_kernels(fast)
+    a = torch.randn(M, K, generator=gen(M + N)).to(a_dtype)
+    w = torch.randn(N, K, generator=gen(K)).to(w_dtype)
+    want = a.double() @ w.double().t()
+    out = torch.empty(M, N, dtype=c_dtype, device=DEV)
+    _ops.gemm(out, a.to(DEV), w.to(DEV))
+    close(out, want, 2e-6 if c_dtype == F32 else 2 ** -8, f"gemm {M}x{N}x{K}")
+    if c_dtype == F32:
+        base = torch.randn(M, N, generator=gen(9))
+        acc = base.clone().to(DEV)
+        _ops.gemm(acc, a.to(DEV), w.to(DEV), accumulate=True)
+        close(acc, want + base.double(), 2e-6, "gemm accumulate")
+
+
+def test_gemm_reference_vectors(_ops):
+    # tests/ops/test_matmul.cpp:90-204
+    W = torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]], device=DEV)
+    X = torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]], device=DEV)
+    out = torch.empty(2, 2, device=DEV)
+    _ops.gemm(out, X, W)
+    assert out.cpu().tolist() == [[14.0, 32.0], [32.0, 77.0]]
+
+
+@pytest.mark.parametrize("fast", [False, True])
+def test_gemm_rows_do_not_depend_on_the_batch(_ops, fast):
+    """A row's result is the same whatever other rows share the launch."""
+    _ops.use_fast_kernels(fast)
+    a = torch.randn(150, 264, generator=gen(3)).to(BF16).to(DEV)
+    w = torch.randn(520, 264, generator=gen(4)).to(BF16).to(DEV)
+    whole = torch.empty(150, 520, dtype=F32, device=DEV)
+    _ops.gemm(whole, a, w)
+    for lo, hi in [(0, 1), (7, 9), (64, 150), (149, 150), (3, 70)]:
+        part = torch.empty(hi - lo, 520, dtype=F32, device=DEV)
+        _ops.gemm(part, a[lo:hi], w)
+        close(part, whole[lo:hi].cpu(), 2e-6, f"rows {lo}:{hi}")
+
+
+def test_gemm_takes_strided_views(_ops):
+    a_full = torch.randn(9, 300, generator=gen(5)).to(BF16).to(DEV)
+    w = torch.randn(40, 128, generator=gen(6)).to(BF16).to(DEV)
+    a = a_full[:, 64:192]                       # dense rows, row stride 300
+    out_full = torch.zeros(9, 100, dtype=BF16, device=DEV)
+    _ops.gemm(out_full[:, 8:48], a, w)
+    close(out_full[:, 8:48], a.double().cpu() @ w.double().cpu().t(), 2 ** -8, "strided gemm")
+    assert out_full[:, :8].abs().max() == 0 and out_full[:, 48:].abs().max() == 0
+
+
+def test_ops_refuse_what_they_do_not_take(_ops):
+    from photon_infer_amd import KernelError
+    with pytest.raises(KernelError, match="GPU only"):
+        _ops.gemm(torch.empty(2, 2), torch.empty(2, 3), torch.empty(2, 3))
+    with pytest.raises(KernelError, match="shapes"):
+        _ops.gemm(torch.empty(2, 2, device=DEV), torch.empty(2, 3, device=DEV), torch.empty(2, 4, device=DEV))
+    with pytest.raises(KernelError, match="head_dim"):
+        _ops.check_attention_sizes(4, 2, 40)
+    with pytest.raises(KernelError, match="head_dim"):
+        _ops.check_attention_sizes(4, 2, 272)
+    with pytest.raises(KernelError, match="multiple"):
+        _ops.check_attention_sizes(6, 4, 64)
+    with pytest.raises(KernelError, match="float32 or bfloat16"):
+        _ops.swiglu(torch.empty(2, 4, dtype=torch.float16, device=DEV), torch.empty(2, 8, dtype=torch.float16, device=DEV))
+
+
+# ------------------------------------------------------------------ rotation + cache write
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("hd,rot,inter", [(16, 16, False), (48, 48, True), (64, 32, False), (128, 128, False), (256, 256, True)])
+def test_rope_kv_write(_ops, dtype, hd, rot, inter):
+    nh, nkv, page = 3, 3 if hd == 48 else 1, 4
+    q_lens, kv_lens = [5, 1, 9], [5, 30, 14]          # a whole prompt, a decode at position 29, a later portion
+    T = sum(q_lens)
+    ctx = attention_ctx(q_lens, kv_lens, dtype)
+    freqs = P.rope_frequencies(rot, 500000.0, dict(rope_type="llama3", factor=8.0, low_freq_factor=1.0,
+                                                    high_freq_factor=4.0, original_max_position_embeddings=16))
+    inv = torch.tensor(freqs, dtype=torch.float64).to(F32).to(DEV)
+    qkv = torch.randn(T, (nh + 2 * nkv) * hd, generator=gen(hd)).to(dtype)
+    dev = qkv.to(DEV)
+    q, k, v = dev[:, :nh * hd], dev[:, nh * hd:(nh + nkv) * hd], dev[:, (nh + nkv) * hd:]
+    pages = 12
+    table = torch.full((3, 8), -1, dtype=torch.int32)
+    order = torch.randperm(pages * 2, generator=gen(7))[: 2 + 8 + 4].tolist()
+    table[0, :2], table[1, :8], table[2, :4] = torch.tensor(order[:2]), torch.tensor(order[2:10]), torch.tensor(order[10:14])
+    kc = torch.zeros(pages * 2, nkv, page, hd, dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    _ops.rope_kv_write(q, k, v, ctx.positions, ctx.req_of_token, (inv, rot, inter), nh, nkv, hd, kc, vc, table.to(DEV), page)
+    pos = ctx.positions.cpu().tolist()
+    rel = 1e-6 if dtype == F32 else 2 ** -8
+    q_want = P.rope(qkv[:, :nh * hd].float().reshape(T, nh, hd), pos, freqs, inter)
+    k_want = P.rope(qkv[:, nh * hd:(nh + nkv) * hd].float().reshape(T, nkv, hd), pos, freqs, inter)
+    v_want = qkv[:, (nh + nkv) * hd:].float().reshape(T, nkv, hd)
+    close(q.reshape(T, nh, hd), q_want, rel, "q")
+    req = ctx.req_of_token.cpu().tolist()
+    written = torch.zeros(pages * 2, page, dtype=torch.bool)
+    for t in range(T):
+        pg, sl = table[req[t], pos[t] // page].item(), pos[t] % page
+        written[pg, sl] = True
+        close(kc[pg, :, sl], k_want[t], rel, f"k of token {t}")
+        assert torch.equal(vc[pg, :, sl].cpu().float(), v_want[t])
+    # nothing else in the pool was touched
+    assert kc.cpu()[~written.unsqueeze(1).expand(-1, nkv, -1)].abs().max() == 0
+
+
+# ------------------------------------------------------------------ attention over pages
+def dense_attention(qs, kvs, q_lens, kv_lens, scale, window):
+    """Plain attention per request: the queries are the last q_len positions of kv_len keys."""
+    outs = []
+    for q, (k, v), n, kv in zip(qs, kvs, q_lens, kv_lens):
+        full_q = torch.zeros(kv, q.shape[1], q.shape[2])
+        full_q[kv - n:] = q
+        outs.append(P.attention(full_q, k, v, scale, window=window)[kv - n:])
+    return torch.cat(outs)
+
+
+ATTN_CASES = [
+    # nh, nkv, hd, page, q_lens, kv_lens, window
+    (4, 2, 16, 4, [5, 9, 17], [5, 9, 17], None),                 # whole prompts
+    (4, 1, 32, 8, [1, 1, 1, 1], [1, 7, 33, 100], None),          # decodes, page edges: 1, 7, 33 = 4 pages + 1
+    (6, 3, 48, 16, [2, 16, 1, 3], [40, 16, 65, 130], None),      # mixed, portions down to two tokens
+    (8, 8, 64, 16, [70], [300], None),                           # a late portion of a long prompt
+    (32, 8, 64, 16, [1, 1], [513, 1200], None),                  # the bench's head layout
+    (2, 1, 128, 16, [33, 1], [33, 200], None),
+    (3, 1, 256, 8, [4, 1], [20, 9], None),
+    (4, 2, 16, 4, [6, 1, 20], [6, 23, 40], 7),                   # a window: edge inside and across portions
+    (4, 4, 80, 16, [1, 5], [90, 37], 16),
+]
+
+
+@pytest.mark.parametrize("case", ATTN_CASES, ids=[f"case{i}" for i in range(len(ATTN_CASES))])
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("fast", [False, True])
+def test_paged_attention(_ops, case, dtype, fast):
+    nh, nkv, hd, page, q_lens, kv_lens, window = case
+    if fast and dtype == F32:
+        pytest.skip("the matrix-core kernels take bfloat16 only")
+    _ops.use_fast_kernels(fast)
+    g = gen(nh * 1000 + hd)
+    scale = 1.0 / math.sqrt(hd)
+    kvs = [(torch.randn(kv, nkv, hd, generator=g).to(dtype).float(), torch.randn(kv, nkv, hd, generator=g).to(dtype).float())
+           for kv in kv_lens]
+    qs = [(torch.randn(n, nh, hd, generator=g) * 2).to(dtype).float() for n in q_lens]
+    paged = PagedKV(kvs, page, dtype, seed=hd)
+    ctx = attention_ctx(q_lens, kv_lens, dtype)
+    q = torch.cat(qs).reshape(-1, nh * hd).to(dtype).to(DEV)
+    out = torch.empty_like(q)
+    _ops.paged_attention(out, q, paged.k, paged.v, paged.table, ctx, nh, nkv, hd, page, scale, window or 0)
+    want = dense_attention(qs, kvs, q_lens, kv_lens, scale, window).reshape(-1, nh * hd)
+    close(out, want, 3e-6 if dtype == F32 else 2 ** -7, "attention")
+
+
+@pytest.mark.parametrize("dtype", [F32, BF16])
+@pytest.mark.parametrize("fast", [False, True])
+def test_attention_finds_one_far_key_among_hundreds(_ops, dtype, fast):
+    """One key far back matches the query strongly: the output must be (nearly) its value.
+    A kernel that drops a page, a split or the first / last key of a range fails this."""
+    if fast and dtype == F32:
+        pytest.skip("the matrix-core kernels take bfloat16 only")
+    _ops.use_fast_kernels(fast)
+    nh, nkv, hd, page = 4, 2, 64, 16
+    g = gen(11)
+    for kv_len, q_len, hot in [(777, 1, 3), (777, 1, 776), (640, 1, 639), (777, 1, 512), (500, 37, 15), (500, 37, 463),
+                               (129, 2, 127)]:
+        k = torch.randn(kv_len, nkv, hd, generator=g) * 0.1
+        v = torch.randn(kv_len, nkv, hd, generator=g)
+        q = torch.randn(q_len, nh, hd, generator=g) * 0.1
+        direction = torch.randn(hd, generator=g)
+        direction = direction / direction.norm() * 8.0
+        k[hot] = direction                                     # |k| = 8
+        q += direction * 2.0                                   # score of the hot key: 16 * 8 / 8 = 16 above the rest
+        paged = PagedKV([(k.to(dtype).float(), v.to(dtype).float())], page, dtype, seed=kv_len)
+        ctx = attention_ctx([q_len], [kv_len], dtype)
+        qd = q.reshape(q_len, nh * hd).to(dtype).to(DEV)
+        out = torch.empty_like(qd)
+        _ops.paged_attention(out, qd, paged.k, paged.v, paged.table, ctx, nh, nkv, hd, page, 1.0 / 8.0, 0)
+        out = out.float().cpu().reshape(q_len, nh, hd)
+        for t in range(q_len):
+            p = kv_len - q_len + t
+            if hot <= p:                                       # visible: its value dominates
+                for h in range(nh):
+                    assert (out[t, h] - v[hot, h // 2].to(dtype).float()).abs().max() < 0.05, (kv_len, q_len, hot, t)
+            else:                                              # not yet visible: it must not leak in
+                want = P.attention(torch.cat([torch.zeros(p, nh, hd), q[t:t + 1].to(dtype).float()]),
+                                   k[:p + 1].to(dtype).float(), v[:p + 1].to(dtype).float(), 1.0 / 8.0)[p]
+                assert (out[t] - want).abs().max() < 0.05
+
+
+# ------------------------------------------------------------------ sampling
+def test_greedy_takes_the_lowest_index_among_equals(_ops):
+    V = 128256
+    l = torch.randn(6, V, generator=gen(12))
+    l[0, 7] = 100.0                                            # tests/model/test_llama_model.cpp:236-249
+    l[1, [70000, 99, 120000]] = 50.0
+    l[2] = 0.0
+    l[3, V - 1] = 60.0
+    l[4, :] = float("-inf"); l[4, 4321] = -5.0
+    out = torch.empty(6, dtype=torch.int32, device=DEV)
+    _ops.sample(out, l.to(DEV))
+    assert out.cpu().tolist()[:5] == [7, 99, 0, V - 1, 4321]
+    assert out[5].item() == P.argmax(l[5])
+
+
+def test_temperature_sampling_matches_the_inverse_cdf(_ops):
+    V = 1001
+    g = gen(13)
+    l = torch.randn(64, V, generator=g) * 3
+    temps = torch.full((64,), 0.8)
+    temps[::7] = 0.0                                           # greedy rows beside sampled rows
+    u = torch.rand(64, generator=g)
+    out = torch.empty(64, dtype=torch.int32, device=DEV)
+    _ops.sample(out, l.to(DEV), temps.to(DEV), u.to(DEV))
+    got = out.cpu().tolist()
+    for r in range(64):
+        if temps[r] == 0:
+            assert got[r] == P.argmax(l[r])
+            continue
+        p = torch.softmax(l[r].double() / 0.8, 0)
+        c = torch.cumsum(p, 0)
+        lo = c[got[r] - 1].item() if got[r] > 0 else 0.0
+        assert lo - 1e-5 <= u[r].item() <= c[got[r]].item() + 1e-5, r
+
+
+def test_temperature_sampling_frequencies_and_limits(_ops):
+    from photon_infer_amd.sampling import uniform_draw
+    l = torch.tensor([[0.0, 1.0, 2.0, -1.0, 0.5]]).expand(4000, 5).contiguous()
+    u = torch.tensor([uniform_draw(123, i) for i in range(4000)])
+    assert 0 < u.min() and u.max() < 1 and abs(u.mean().item() - 0.5) < 0.02
+    out = torch.empty(4000, dtype=torch.int32, device=DEV)
+    _ops.sample(out, l.to(DEV), torch.full((4000,), 0.8, device=DEV), u.to(DEV))
+    freq = torch.bincount(out.cpu().long(), minlength=5).float() / 4000
+    assert (freq - torch.softmax(l[0] / 0.8, 0)).abs().max() < 0.025
+    # a tiny temperature is the argmax; u near 1 still lands on a token with p > 0
+    _ops.sample(out[:2], l[:2].to(DEV), torch.full((2,), 1e-4, device=DEV), torch.tensor([0.3, 0.9999999], device=DEV))
+    assert out[:2].cpu().tolist() == [2, 2]
