@@ -155,4 +155,4 @@ def build_module(module: str, force: bool = False, quiet: bool = False) -> str:
 
 
 def build_all(force: bool = True) -> List[str]:
-    return [build_module(m, force=force) for m in MODULES]
+    return [build_module(m, force=force) for m in MODULES if MODULES[m]]

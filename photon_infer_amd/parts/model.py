@@ -82,9 +82,13 @@ def plan_cache(spec: ModelSpec) -> CachePlan:
     by_window: Dict[Optional[int], List[Tuple[int, KVCacheSpec]]] = {}
     states: List[Tuple[int, StateSpec]] = []
     for i, e in enumerate(spec.run_order):
+        mixer = spec.layers[e.layer][1].mixer
         if e.cache_of is not None:
             continue
-        need = spec.layers[e.layer][1].mixer.cache_spec()
+        if not getattr(mixer, "own_kv", True):
+            raise ConfigError(f"run order entry {i}: layer {e.layer} writes no keys or values of its own and "
+                              f"must name the entry whose cache it reads")
+        need = mixer.cache_spec()
         if isinstance(need, KVCacheSpec):
             by_window.setdefault(need.window, []).append((i, need))
         elif isinstance(need, StateSpec):

@@ -1,0 +1,140 @@
+"""Generation through the entry points: Python engine and command line."""
+import json
+import os
+import subprocess
+
+import pytest
+import torch
+
+import plain_llama as P
+from tiny_models import ALL, make_model_dir, random_tokens
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def model_dirs(tmp_path_factory):
+    root = tmp_path_factory.mktemp("models")
+    return {name: make_model_dir(root, name, seed=21) for name in ("A", "B")}
+
+
+def engine(model_dir, name, **kw):
+    from photon_infer_amd import ContinuousBatchEngine
+    opts = dict(dtype="float32", block_size=ALL[name][1]["block_size"], num_blocks=128, max_batch=4)
+    opts.update(kw)
+    return ContinuousBatchEngine(model_dir, **opts)
+
+
+def test_greedy_generation_equals_the_plain_implementation(model_dirs):
+    # BASELINE workload of the first tiny model: prompts of 5, 9 and 17 tokens, 8 greedy tokens each
+    cfg, W = P.read_model_folder(model_dirs["A"])
+    prompts = [random_tokens(n, 256, 30 + n) for n in (5, 9, 17)]
+    want = [P.greedy_generate(cfg, W, p, 8) for p in prompts]
+    eng = engine(model_dirs["A"], "A")
+    assert eng.generate(prompts, max_new_tokens=8, ignore_eos=True) == want
+    # alone, one at a time: the same tokens as batched with the others
+    for p, w in zip(prompts, want):
+        assert engine(model_dirs["A"], "A").generate([p], max_new_tokens=8, ignore_eos=True) == [w]
+    assert eng.runner.cache.num_live == 0 and eng.runner.cache.free_pages() == 128
+
+
+def test_greedy_generation_in_bfloat16_follows_the_plain_arg_max(model_dirs):
+    cfg, W = P.read_model_folder(model_dirs["B"])
+    prompts = [random_tokens(n, 384, 40 + n) for n in (1, 7, 33)]
+    outs = engine(model_dirs["B"], "B", dtype="bfloat16", chunk_size=16).generate(prompts, max_new_tokens=10, ignore_eos=True)
+    for p, out in zip(prompts, outs):
+        seq = list(p)
+        assert len(out) == 10
+        for tok in out:
+            ref = P.llama_forward(cfg, W, seq)[-1]
+            emu = P.llama_forward(cfg, W, seq, act_round=P.bf16_round)[-1]
+            slack = 3.0 * (emu - ref).abs().max().item()
+            assert ref[tok].item() >= ref.max().item() - 2 * slack, (seq, tok)
+            seq.append(tok)
+
+
+def test_chunked_prefill_beside_decodes_with_temperature(model_dirs):
+    # BASELINE workload of the second tiny model: prompts 1, 7, 33, 64, 100 in 16-token chunks
+    # beside decodes, 12 tokens each at temperature 0.8
+    prompts = [random_tokens(n, 384, 50 + n) for n in (1, 7, 33, 64, 100)]
+
+    def run(order, **kw):
+        eng = engine(model_dirs["B"], "B", chunk_size=16, max_step_tokens=40, **kw)
+        ids = {i: eng.add_request(prompts[i], 12, temperature=0.8, seed=1000 + i, ignore_eos=True) for i in order}
+        eng.run_until_complete()
+        return {i: eng.get_result(ids[i]) for i in order}, eng
+
+    a, eng = run([0, 1, 2, 3, 4])
+    assert all(len(v) == 12 for v in a.values())
+    assert eng.get_stats().num_steps > 12                       # prompts were cut into portions
+    b, _ = run([4, 2, 0, 3, 1])                                 # another admission order, other batches
+    c, _ = run([3], max_batch=1)                                # alone
+    assert a == b and c[3] == a[3]                              # same (seed, request) => same tokens
+    # and the draws are those of the plain sampler on the plain logits
+    cfg, W = P.read_model_folder(model_dirs["B"])
+    from photon_infer_amd.sampling import uniform_draw
+    seq = list(prompts[1])
+    for k, tok in enumerate(a[1]):
+        logits = P.llama_forward(cfg, W, seq)[-1]
+        assert tok == P.sample_temperature(logits, 0.8, uniform_draw(1001, k))
+        seq.append(tok)
+
+
+def test_out_of_pages_preempts_and_recomputes_to_the_same_tokens(model_dirs):
+    prompts = [random_tokens(n, 256, 60 + n) for n in (20, 20, 20)]
+    roomy = engine(model_dirs["A"], "A")
+    want = roomy.generate(prompts, max_new_tokens=30, ignore_eos=True)
+    tight = engine(model_dirs["A"], "A", num_blocks=30)        # 120 tokens of cache for 3 x 50
+    got = tight.generate(prompts, max_new_tokens=30, ignore_eos=True)
+    assert tight.get_stats().num_preemptions > 0
+    assert got == want
+    assert tight.runner.cache.free_pages() == 30
+    tight.runner.cache.check_invariants()
+
+
+def test_eos_ends_a_request_and_limits_hold(model_dirs, tmp_path):
+    cfg, W = P.read_model_folder(model_dirs["A"])
+    prompt = random_tokens(9, 256, 70)
+    free_run = P.greedy_generate(cfg, W, prompt, 8)
+    eos = free_run[3]
+    d = str(tmp_path / "with_eos")
+    os.makedirs(d)
+    json.dump(dict(cfg, eos_token_id=[eos, 999999]), open(os.path.join(d, "config.json"), "w"))
+    os.symlink(os.path.join(model_dirs["A"], "model.safetensors"), os.path.join(d, "model.safetensors"))
+    eng = engine(d, "A")
+    rid = eng.add_request(prompt, 8)
+    eng.run_until_complete()
+    req = eng.get_request(rid)
+    assert req.generated_tokens == free_run[:free_run.index(eos) + 1] and req.finish_reason == "eos"
+    from photon_infer_amd import RequestError
+    with pytest.raises(RequestError, match="vocabulary"):
+        eng.add_request([1, 2, 256])
+    with pytest.raises(RequestError, match="longer"):
+        eng.add_request([1] * 129)
+
+
+def test_command_line(model_dirs, tmp_path):
+    cfg, W = P.read_model_folder(model_dirs["A"])
+    prompt = random_tokens(6, 256, 80)
+    want = P.greedy_generate(cfg, W, prompt, 5)
+    proc = subprocess.run(
+        [os.path.join(ROOT, "bin", "llama_infer"), model_dirs["A"], "--dtype", "fp32", "--prompt-ids",
+         ",".join(map(str, prompt)), "--max-new-tokens", "5", "--temperature", "0", "--block-size", "4", "--ignore-eos"],
+        capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "PhotonInfer - LLaMA Inference Demo" in proc.stdout and "tokens/s" in proc.stdout
+    assert f"Generated ids: {','.join(map(str, want))}" in proc.stdout
+    # random-weights mode from a bare config.json, text prompt through a tokenizer file
+    import base64
+    (tmp_path / "cfg").mkdir()
+    json.dump(ALL["A"][0], open(tmp_path / "cfg" / "config.json", "w"))
+    (tmp_path / "tok.model").write_text("".join(f"{base64.b64encode(bytes([b])).decode()} {b}\n" for b in range(256)))
+    cfg_small = dict(ALL["A"][0], vocab_size=128256)
+    json.dump(cfg_small, open(tmp_path / "cfg" / "config.json", "w"))
+    proc = subprocess.run(
+        [os.path.join(ROOT, "bin", "llama_infer"), str(tmp_path / "cfg"), str(tmp_path / "tok.model"), "cuda",
+         "--random-weights", "--seed", "3", "--prompt", "hi there", "--max-new-tokens", "4"],
+        capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert "User: hi there" in proc.stdout and "Prompt tokens: 9" in proc.stdout and "Assistant:" in proc.stdout
