@@ -23,7 +23,7 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
     float scale, int window, long num_pages) {
   __shared__ float qs[PI_MAX_HEAD_DIM];
   __shared__ float ps[PI_WAVE];
-  __shared__ long rowoff[PI_WAVE];
+  __shared__ long voff[PI_WAVE];   // values are stored [page, kv_head, head_dim, slot]
   const long t = blockIdx.x;
   const int h = blockIdx.y;
   const int lane = threadIdx.x;
@@ -39,12 +39,13 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
   for (int k0 = lo; k0 <= p; k0 += PI_WAVE) {
     const int key = k0 + lane;
     float s = -INFINITY;
-    long off = -1;
+    long off = -1, vo = -1;
     if (key <= p) {
       const int blk = key / page_size;
       const long page = blk < table_width ? bt[blk] : -1;
       if (page >= 0 && page < num_pages) {
         off = ((page * nkv + g) * page_size + (key % page_size)) * hd;
+        vo = (page * nkv + g) * (long)page_size * hd + (key % page_size);
         const T* kr = k_cache + off;
         float dot = 0.f;
         for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], to_float(kr[d]), dot);
@@ -58,20 +59,20 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
     const float corr = expf(m - m_new);
     l = l * corr + wave_sum(pe);
     ps[lane] = pe;
-    rowoff[lane] = off;
+    voff[lane] = vo;
 #pragma unroll
     for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) acc[i] *= corr;
     __syncthreads();
     const int nk = (p - k0 + 1) < PI_WAVE ? (p - k0 + 1) : PI_WAVE;
     for (int kk = 0; kk < nk; ++kk) {
-      const long o2 = rowoff[kk];
+      const long o2 = voff[kk];
       if (o2 < 0) continue;
       const T* vr = v_cache + o2;
       const float pk = ps[kk];
 #pragma unroll
       for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
         const int d = lane + i * PI_WAVE;
-        if (d < hd) acc[i] = fmaf(pk, to_float(vr[d]), acc[i]);
+        if (d < hd) acc[i] = fmaf(pk, to_float(vr[(long)d * page_size]), acc[i]);
       }
     }
     m = m_new;

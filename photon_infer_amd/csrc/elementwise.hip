@@ -73,29 +73,34 @@ extern "C" int pi_rmsnorm(void* out, int out_dtype, const float* x, const int* r
 }
 
 // ------------------------------------------------------------------ SwiGLU
-// out[t, i] = g / (1 + exp(-g)) * u with g = gu[t, i], u = gu[t, I + i]; float32 math.
+// out[t, i] = g / (1 + exp(-g)) * u; float32 math.  Layout of gu [T, 2I]:
+//   block == 0: gate in columns [0, I), up in [I, 2I);
+//   block == b: gate and up interleaved in blocks of b columns (gate block, up block, ...).
 template <typename T>
-__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, long total, int I) {
+__global__ void swiglu_kernel(T* __restrict__ out, const T* __restrict__ gu, long total, int I, int block) {
   const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
   if (idx >= total) return;
   const long t = idx / I;
   const int i = (int)(idx - t * I);
-  const float g = to_float(gu[t * 2 * I + i]);
-  const float u = to_float(gu[t * 2 * I + I + i]);
+  const long gi = block ? (long)(i / block) * 2 * block + i % block : i;
+  const long ui = block ? gi + block : (long)I + i;
+  const float g = to_float(gu[t * 2 * I + gi]);
+  const float u = to_float(gu[t * 2 * I + ui]);
   out[idx] = from_float<T>(g / (1.0f + expf(-g)) * u);
 }
 
-extern "C" int pi_swiglu(void* out, const void* gu, int dtype, int T, int I, hipStream_t stream) {
+extern "C" int pi_swiglu(void* out, const void* gu, int dtype, int T, int I, int block, hipStream_t stream) {
   PI_REQUIRE(T >= 0 && I > 0, "swiglu: bad sizes T=%d I=%d", T, I);
+  PI_REQUIRE(block >= 0 && (block == 0 || I % block == 0), "swiglu: interleave block %d does not divide %d", block, I);
   if (T == 0) return 0;
   const long total = (long)T * I;
   const int threads = 256;
   const long blocks = (total + threads - 1) / threads;
   PI_REQUIRE(blocks < 2147483647L, "swiglu: too many elements (%ld)", total);
   if (dtype == PI_F32)
-    hipLaunchKernelGGL(swiglu_kernel<float>, dim3((unsigned)blocks), dim3(threads), 0, stream, (float*)out, (const float*)gu, total, I);
+    hipLaunchKernelGGL(swiglu_kernel<float>, dim3((unsigned)blocks), dim3(threads), 0, stream, (float*)out, (const float*)gu, total, I, block);
   else if (dtype == PI_BF16)
-    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3((unsigned)blocks), dim3(threads), 0, stream, (bf16_t*)out, (const bf16_t*)gu, total, I);
+    hipLaunchKernelGGL(swiglu_kernel<bf16_t>, dim3((unsigned)blocks), dim3(threads), 0, stream, (bf16_t*)out, (const bf16_t*)gu, total, I, block);
   else
     return pi_fail("swiglu: unsupported dtype %d", dtype);
   return pi_check_launch("swiglu");
@@ -105,7 +110,9 @@ extern "C" int pi_swiglu(void* out, const void* gu, int dtype, int T, int I, hip
 // One wave per (token, head).  Heads 0..nh-1 are queries (rotated in place); then, when
 // the layer writes its cache, nkv key heads (rotated, stored to the page of the token's
 // position) and nkv value heads (stored as they are).
-// Cache layout: [page, kv_head, slot_in_page, head_dim].
+// Cache layout: keys [page, kv_head, slot_in_page, head_dim]; values transposed,
+// [page, kv_head, head_dim, slot_in_page], so that the keys of one page are contiguous for a
+// fixed feature - the order in which the matrix-core attention kernels contract them.
 // angle = float(pos) * inv_freq[j]; pair j is (x[j], x[j + R/2]) or, interleaved,
 // (x[2j], x[2j+1]); (a, b) <- (a cos - b sin, a sin + b cos).  Dims >= R are copied.
 template <typename T>
@@ -137,9 +144,10 @@ __global__ void rope_kv_write_kernel(T* __restrict__ q, long q_stride, const T* 
     if (page < 0 || page >= num_pages) return;  // the host checks tables; never write outside the pool
     const long off = ((page * nkv + g) * page_size + (pos % page_size)) * hd;
     if (is_v) {
-      src = v + t * v_stride + (long)g * hd;
-      dst = v_cache + off;
-      rotate = false;
+      const T* vs = v + t * v_stride + (long)g * hd;
+      T* vd = v_cache + (page * nkv + g) * (long)page_size * hd + (pos % page_size);
+      for (int d = lane; d < hd; d += PI_WAVE) vd[(long)d * page_size] = vs[d];
+      return;
     } else {
       src = k + t * k_stride + (long)g * hd;
       dst = k_cache + off;

@@ -69,13 +69,13 @@ class ModelRunner:
         self.cache = CacheManager([g.window for g in self.plan.groups], self.page_size, num_pages,
                                   o.max_batch, self.max_model_len)
         self.states = StateSlots(self.plan.states, o.max_batch, self.device)
-        # one K and one V pool per run-order entry that owns pages: [pages, kv_heads, page, head_dim]
+        # one K and one V pool per run-order entry that owns pages: keys [pages, kv_heads, page,
+        # head_dim], values [pages, kv_heads, head_dim, page] (the layout the kernels contract in)
         pools: Dict[int, tuple] = {}
         for g in self.plan.groups:
             for entry, (nkv, hd) in zip(g.entries, g.kv_shapes):
-                shape = (num_pages, nkv, self.page_size, hd)
-                pools[entry] = (torch.zeros(shape, dtype=self.dtype, device=self.device),
-                                torch.zeros(shape, dtype=self.dtype, device=self.device))
+                pools[entry] = (torch.zeros((num_pages, nkv, self.page_size, hd), dtype=self.dtype, device=self.device),
+                                torch.zeros((num_pages, nkv, hd, self.page_size), dtype=self.dtype, device=self.device))
         self.layer_caches: List[LayerCache] = []
         for i, e in enumerate(self.spec.run_order):
             owner = i if e.cache_of is None else e.cache_of

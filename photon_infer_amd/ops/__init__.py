@@ -119,13 +119,35 @@ def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float
               _dt(weight), float(eps), M, D, _stream())
 
 
-def swiglu(out: torch.Tensor, gate_up: torch.Tensor) -> None:
-    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i]."""
+def swiglu(out: torch.Tensor, gate_up: torch.Tensor, block: int = 0) -> None:
+    """out[t, i] = silu(gate) * up.  ``block`` = 0: gate in columns [0, I), up in [I, 2I);
+    ``block`` = b: gate and up interleaved in blocks of b columns."""
     _gpu(out, gate_up)
     T, I = out.shape
     if gate_up.shape != (T, 2 * I) or gate_up.dtype != out.dtype or not (out.is_contiguous() and gate_up.is_contiguous()):
         raise KernelError(f"swiglu: expected gate_up [{T}, {2 * I}] of {out.dtype}, got {tuple(gate_up.shape)} {gate_up.dtype}")
-    _lib.call("core", "pi_swiglu", out.data_ptr(), gate_up.data_ptr(), _dt(out), T, I, _stream())
+    if block < 0 or (block and I % block):
+        raise KernelError(f"swiglu: interleave block {block} does not divide {I}")
+    _lib.call("core", "pi_swiglu", out.data_ptr(), gate_up.data_ptr(), _dt(out), T, I, int(block), _stream())
+
+
+def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate_up: torch.Tensor, block: int = 0) -> None:
+    """out[M, I] = silu(a @ Wg^T) * (a @ Wu^T) where ``w_gate_up`` [2I, K] holds the gate and
+    up rows in halves (``block`` 0) or interleaved in blocks of ``block`` rows.  With bfloat16
+    operands and blocks of 16 the product and the activation are one kernel."""
+    _gpu(out, a, w_gate_up)
+    M, I = out.shape
+    if w_gate_up.shape[0] != 2 * I or a.shape != (M, w_gate_up.shape[1]) or out.dtype != a.dtype:
+        raise KernelError(f"gemm_swiglu: shapes do not agree: a {tuple(a.shape)}, w {tuple(w_gate_up.shape)}, out {tuple(out.shape)}")
+    if M == 0:
+        return
+    if _FAST and block == 16 and a.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and out.is_contiguous():
+        from . import fast
+        if fast.gemm_swiglu(out, a, w_gate_up, M, 2 * I, a.shape[1], _rows(a, "gemm a"), _rows(w_gate_up, "gemm w")):
+            return
+    gu = torch.empty((M, 2 * I), dtype=a.dtype, device=a.device)
+    gemm(gu, a, w_gate_up)
+    swiglu(out, gu, block)
 
 
 def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, accumulate: bool = False) -> None:
@@ -151,8 +173,11 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, accumulate: bool =
 
 
 def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, hd: int, page_size: int, dtype) -> int:
-    if k_cache.shape != v_cache.shape or k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (nkv, page_size, hd):
-        raise KernelError(f"cache: expected [pages, {nkv}, {page_size}, {hd}], got {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
+    """Keys [pages, kv_heads, page, head_dim]; values transposed, [pages, kv_heads, head_dim, page]."""
+    if (k_cache.dim() != 4 or tuple(k_cache.shape[1:]) != (nkv, page_size, hd)
+            or tuple(v_cache.shape) != (k_cache.shape[0], nkv, hd, page_size)):
+        raise KernelError(f"cache: expected keys [pages, {nkv}, {page_size}, {hd}] and values [pages, {nkv}, {hd}, {page_size}], "
+                          f"got {tuple(k_cache.shape)} / {tuple(v_cache.shape)}")
     if k_cache.dtype != dtype or v_cache.dtype != dtype or not (k_cache.is_contiguous() and v_cache.is_contiguous()):
         raise KernelError(f"cache: must be contiguous {dtype}, got {k_cache.dtype}")
     return k_cache.shape[0]

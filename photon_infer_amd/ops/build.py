@@ -26,9 +26,9 @@ CSRC_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__
 # matrix-core kernels that only the bfloat16 path uses.
 MODULES: Dict[str, List[str]] = {
     "core": ["elementwise.hip", "gemm_general.hip", "attention_general.hip", "sampling.hip"],
-    "bf16": [],
+    "bf16": ["gemm_mfma.hip", "gemm_skinny.hip", "attention_mfma.hip", "attention_decode.hip"],
 }
-HEADERS = ["common.h", "mfma.h"]
+HEADERS = ["common.h", "mfma.h", "attention_mfma.h"]
 
 ARCH = "gfx950"
 HIPCC_FLAGS = [

@@ -2,17 +2,170 @@
 
 Each function returns True when it ran the operation and False when the sizes are not
 ones its kernels take, in which case the caller uses the general kernel.
+
+Which kernel takes what:
+  * matrix products: K and the row strides multiples of 8, 16-byte aligned operands;
+    up to 64 rows go to the weight-streaming kernel (k split over blocks where the output
+    is narrow), more rows to the 128 x 128 tile kernel;
+  * attention: head_dim 64 or 128, pages of a multiple of 16 tokens; a batch of single
+    tokens with at most 16 heads per kv head goes to the key-split decode kernel, any other
+    batch to the tile kernel.
 """
 from __future__ import annotations
 
+from typing import Dict, Optional
+
+import numpy as np
+import torch
+
+from . import _lib
+
+EPI_BF16, EPI_F32, EPI_ACCUM, EPI_SWIGLU = 0, 1, 2, 3
+SKINNY_MAX_ROWS = 64
+ROWS_PER_BLOCK = 32            # weight rows per block of the skinny kernel
+TARGET_BLOCKS = 512            # blocks wanted in flight to keep HBM busy
+GEMM_PART_FLOATS = 4 << 20     # k-split partial sums of the skinny kernel
+GEMM_COUNTERS = 8192
+ATTN_PART_FLOATS = 4 << 20     # key-split partial results of decode attention
+ATTN_COUNTERS = 1 << 16
+MAX_DECODE_SPLITS = 64
+
+
+class _Workspace:
+    """Scratch the kernels share on one device: partial sums and self-resetting counters.
+    Kernels on one stream run one after another, so one set is enough."""
+
+    def __init__(self, device):
+        self.gemm_part = torch.empty(GEMM_PART_FLOATS, dtype=torch.float32, device=device)
+        self.gemm_counters = torch.zeros(GEMM_COUNTERS, dtype=torch.int32, device=device)
+        self.attn_part = torch.empty(ATTN_PART_FLOATS, dtype=torch.float32, device=device)
+        self.attn_counters = torch.zeros(ATTN_COUNTERS, dtype=torch.int32, device=device)
+
+
+_WORKSPACES: Dict[torch.device, _Workspace] = {}
+
+
+def workspace(device) -> _Workspace:
+    ws = _WORKSPACES.get(device)
+    if ws is None:
+        ws = _WORKSPACES[device] = _Workspace(device)
+    return ws
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _gemm_ok(a, w, K, lda, ldw) -> bool:
+    return K % 8 == 0 and lda % 8 == 0 and ldw % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+
+
+def _skinny_splits(M: int, N: int, K: int) -> int:
+    groups = -(-N // ROWS_PER_BLOCK)
+    splits = max(1, min(-(-TARGET_BLOCKS // groups), K // 256))
+    while splits > 1 and splits * M * N > GEMM_PART_FLOATS:
+        splits -= 1
+    return splits if groups <= GEMM_COUNTERS else 1
+
+
+def _run_gemm(out, epilogue: int, ldc: int, a, w, M: int, N: int, K: int, lda: int, ldw: int) -> None:
+    if M <= SKINNY_MAX_ROWS:
+        splits = 1 if epilogue == EPI_SWIGLU else _skinny_splits(M, N, K)
+        ws = workspace(a.device)
+        _lib.call("bf16", "pi_gemm_skinny", out.data_ptr(), epilogue, ldc, a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K,
+                  splits, ws.gemm_part.data_ptr(), ws.gemm_part.numel(), ws.gemm_counters.data_ptr(),
+                  ws.gemm_counters.numel(), _stream())
+    else:
+        _lib.call("bf16", "pi_gemm_mfma", out.data_ptr(), epilogue, ldc, a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K,
+                  _stream())
+
 
 def gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc) -> bool:
-    return False
+    if not _gemm_ok(a, w, K, lda, ldw):
+        return False
+    if accumulate:
+        epilogue = EPI_ACCUM
+    elif out.dtype == torch.bfloat16:
+        epilogue = EPI_BF16
+    elif out.dtype == torch.float32:
+        epilogue = EPI_F32
+    else:
+        return False
+    _run_gemm(out, epilogue, ldc, a, w, M, N, K, lda, ldw)
+    return True
+
+
+def gemm_swiglu(out, a, w, M, N, K, lda, ldw) -> bool:
+    """``w`` [N = 2I, K] with gate / up rows interleaved in blocks of 16; out [M, I] bfloat16."""
+    if not _gemm_ok(a, w, K, lda, ldw) or N % 32 or out.dtype != torch.bfloat16:
+        return False
+    _run_gemm(out, EPI_SWIGLU, out.stride(0), a, w, M, N, K, lda, ldw)
+    return True
+
+
+# ----------------------------------------------------------------------------- attention
+def attention_tile_rows(num_heads: int, num_kv_heads: int, head_dim: int) -> int:
+    return _lib.load("bf16").pi_attention_tile_rows(num_heads, num_kv_heads, head_dim)
+
+
+def _tiles(ctx, tile_rows: int, device):
+    """Work list of the tile kernel: (request, first token) of every tile; cached on the step."""
+    cache = getattr(ctx, "_attention_tiles", None)
+    if cache is None:
+        cache = {}
+        try:
+            ctx._attention_tiles = cache
+        except AttributeError:
+            pass
+    hit = cache.get(tile_rows)
+    if hit is None:
+        req, q0 = [], []
+        for r, n in enumerate(ctx.q_lens):
+            for start in range(0, n, tile_rows):
+                req.append(r)
+                q0.append(start)
+        host = np.asarray([req, q0], np.int32)
+        dev = torch.from_numpy(host).to(device)
+        hit = cache[tile_rows] = (dev[0], dev[1], len(req))
+    return hit
+
+
+def decode_splits(R: int, num_kv_heads: int, max_kv_len: Optional[int] = None) -> int:
+    """Key ranges per (request, kv head): enough waves to fill the chip, no more than the
+    keys are worth."""
+    splits = max(1, min(MAX_DECODE_SPLITS, -(-1024 // (R * num_kv_heads))))
+    if max_kv_len is not None:
+        splits = min(splits, max(1, -(-max_kv_len // 64)))
+    return splits
 
 
 def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
                     page_size, scale, window, pages) -> bool:
-    return False
+    if head_dim not in (64, 128) or page_size % 16 or q.data_ptr() % 16 or q.stride(0) % 8 or out.stride(0) % 4:
+        return False
+    G = num_heads // num_kv_heads
+    R = ctx.R
+    if ctx.all_decode and G <= 16:
+        splits = getattr(ctx, "decode_splits_fixed", None) or decode_splits(R, num_kv_heads, ctx.max_kv_len)
+        ws = workspace(q.device)
+        while splits > 1 and R * num_heads * splits * (head_dim + 4) > ws.attn_part.numel():
+            splits -= 1
+        if R * num_kv_heads <= ws.attn_counters.numel():
+            _lib.call("bf16", "pi_attention_decode", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
+                      k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+                      ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), R, num_heads, num_kv_heads, head_dim, page_size,
+                      float(scale), int(window), pages, splits, ws.attn_part.data_ptr(), ws.attn_part.numel(),
+                      ws.attn_counters.data_ptr(), ws.attn_counters.numel(), _stream())
+            return True
+    tile_rows = attention_tile_rows(num_heads, num_kv_heads, head_dim)
+    if tile_rows < 1:
+        return False
+    tile_req, tile_q0, num_tiles = _tiles(ctx, tile_rows, q.device)
+    _lib.call("bf16", "pi_attention_prefill_mfma", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
+              k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+              ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(), num_tiles,
+              num_heads, num_kv_heads, head_dim, page_size, float(scale), int(window), pages, _stream())
+    return True
 
 
 def plan_attention(q_lens, kv_lens) -> dict:

@@ -91,7 +91,7 @@ class LayerCache:
 
     group: int = -1                       # cache group of the pages (-1: no pages)
     k: Optional[torch.Tensor] = None      # [pages, kv_heads, page_size, head_dim]
-    v: Optional[torch.Tensor] = None
+    v: Optional[torch.Tensor] = None      # [pages, kv_heads, head_dim, page_size]
     page_size: int = 0
     writes: bool = True                   # False: reads another entry's cache
     state: Optional[torch.Tensor] = None  # [max_slots, *StateSpec.shape]

@@ -16,6 +16,8 @@ from ..errors import UnsupportedModelError
 from ..weights.loader import TensorSpec
 from .base import FEED_FORWARDS, FeedForward, StepContext
 
+INTERLEAVE = 16   # rows of a matrix-core tile
+
 
 class SwiGLU(FeedForward):
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
@@ -36,16 +38,23 @@ class SwiGLU(FeedForward):
         super().load(tensors, dtype, device)
         g, u = tensors["gate_proj.weight"], tensors["up_proj.weight"]
         common = torch.float32 if torch.float32 in (g.dtype, u.dtype) else g.dtype
-        # one projection for gate and up: rows [gate | up]
-        self.w_gate_up = torch.cat([g.to(common), u.to(common)], dim=0).contiguous()
+        g, u = g.to(common), u.to(common)
+        I = self.intermediate_size
+        if common == torch.bfloat16 and I % INTERLEAVE == 0:
+            # one projection for gate and up, rows interleaved in blocks of 16 (gate block, up
+            # block, ...): the matrix-core kernels then hold a feature's gate and up value in
+            # the same lane and apply the activation before anything is stored
+            self.interleave = INTERLEAVE
+            self.w_gate_up = torch.stack([g.view(I // INTERLEAVE, INTERLEAVE, -1), u.view(I // INTERLEAVE, INTERLEAVE, -1)],
+                                         dim=1).reshape(2 * I, -1).contiguous()
+        else:
+            self.interleave = 0                      # rows [gate | up]
+            self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
         self.w_down = tensors["down_proj.weight"]
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
-        T = h.shape[0]
-        gu = torch.empty((T, 2 * self.intermediate_size), dtype=self.dtype, device=h.device)
-        ops.gemm(gu, h, self.w_gate_up)
-        act = torch.empty((T, self.intermediate_size), dtype=self.dtype, device=h.device)
-        ops.swiglu(act, gu)
+        act = torch.empty((h.shape[0], self.intermediate_size), dtype=self.dtype, device=h.device)
+        ops.gemm_swiglu(act, h, self.w_gate_up, self.interleave)
         ops.gemm(x, act, self.w_down, accumulate=True)
 
 

@@ -43,7 +43,7 @@ class PagedKV:
         self.table = torch.full((len(seqs), width), -1, dtype=torch.int32)
         # unused pages hold large values: a read outside a request's keys shows
         self.k = torch.full((total, nkv, page_size, hd), 1e4, dtype=torch.float32)
-        self.v = torch.full((total, nkv, page_size, hd), -1e4, dtype=torch.float32)
+        self.v = torch.full((total, nkv, hd, page_size), -1e4, dtype=torch.float32)   # values are kept transposed
         it = iter(order)
         for r, (k, v) in enumerate(seqs):
             for b in range(blocks[r]):
@@ -51,7 +51,7 @@ class PagedKV:
                 self.table[r, b] = page
                 n = min(page_size, k.shape[0] - b * page_size)
                 self.k[page, :, :n] = k[b * page_size: b * page_size + n].transpose(0, 1)
-                self.v[page, :, :n] = v[b * page_size: b * page_size + n].transpose(0, 1)
+                self.v[page, :, :, :n] = v[b * page_size: b * page_size + n].permute(1, 2, 0)
         self.k = self.k.to(dtype).to(DEV)
         self.v = self.v.to(dtype).to(DEV)
         self.table = self.table.to(DEV)

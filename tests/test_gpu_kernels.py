@@ -110,6 +110,26 @@ def test_gemm(_ops, M, N, K, a_dtype, w_dtype, c_dtype, fast):
         close(acc, want + base.double(), 2e-6, "gemm accumulate")
 
 
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 64, 65, 200])
+@pytest.mark.parametrize("I,K", [(176, 64), (272, 128), (8192 // 8, 2048 // 8)])
+def test_gemm_with_swiglu_in_the_epilogue(_ops, M, I, K):
+    """Gate and up rows interleaved by 16: product and activation in one kernel."""
+    a = torch.randn(M, K, generator=gen(M)).to(BF16)
+    g = (torch.randn(I, K, generator=gen(I)) * 0.3).to(BF16)
+    u = (torch.randn(I, K, generator=gen(K)) * 0.3).to(BF16)
+    w_il = torch.stack([g.view(I // 16, 16, K), u.view(I // 16, 16, K)], dim=1).reshape(2 * I, K).contiguous()
+    want = P.swiglu(a.double() @ g.double().t(), a.double() @ u.double().t())
+    for fast in (True, False):
+        _ops.use_fast_kernels(fast)
+        out = torch.empty(M, I, dtype=BF16, device=DEV)
+        _ops.gemm_swiglu(out, a.to(DEV), w_il.to(DEV), 16)
+        close(out, want, 2 ** -7, f"fused swiglu fast={fast}")
+    halves = torch.cat([g, u]).to(DEV)
+    out = torch.empty(M, I, dtype=BF16, device=DEV)
+    _ops.gemm_swiglu(out, a.to(DEV), halves, 0)
+    close(out, want, 2 ** -7, "swiglu on halves")
+
+
 def test_gemm_reference_vectors(_ops):
     # tests/ops/test_matmul.cpp:90-204
     W = torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]], device=DEV)
@@ -178,7 +198,7 @@ def test_rope_kv_write(_ops, dtype, hd, rot, inter):
     order = torch.randperm(pages * 2, generator=gen(7))[: 2 + 8 + 4].tolist()
     table[0, :2], table[1, :8], table[2, :4] = torch.tensor(order[:2]), torch.tensor(order[2:10]), torch.tensor(order[10:14])
     kc = torch.zeros(pages * 2, nkv, page, hd, dtype=dtype, device=DEV)
-    vc = torch.zeros_like(kc)
+    vc = torch.zeros(pages * 2, nkv, hd, page, dtype=dtype, device=DEV)
     _ops.rope_kv_write(q, k, v, ctx.positions, ctx.req_of_token, (inv, rot, inter), nh, nkv, hd, kc, vc, table.to(DEV), page)
     pos = ctx.positions.cpu().tolist()
     rel = 1e-6 if dtype == F32 else 2 ** -8
@@ -192,9 +212,10 @@ def test_rope_kv_write(_ops, dtype, hd, rot, inter):
         pg, sl = table[req[t], pos[t] // page].item(), pos[t] % page
         written[pg, sl] = True
         close(kc[pg, :, sl], k_want[t], rel, f"k of token {t}")
-        assert torch.equal(vc[pg, :, sl].cpu().float(), v_want[t])
+        assert torch.equal(vc[pg, :, :, sl].cpu().float(), v_want[t])
     # nothing else in the pool was touched
     assert kc.cpu()[~written.unsqueeze(1).expand(-1, nkv, -1)].abs().max() == 0
+    assert vc.cpu().permute(0, 1, 3, 2)[~written.unsqueeze(1).expand(-1, nkv, -1)].abs().max() == 0
 
 
 # ------------------------------------------------------------------ attention over pages
@@ -219,6 +240,14 @@ ATTN_CASES = [
     (3, 1, 256, 8, [4, 1], [20, 9], None),
     (4, 2, 16, 4, [6, 1, 20], [6, 23, 40], 7),                   # a window: edge inside and across portions
     (4, 4, 80, 16, [1, 5], [90, 37], 16),
+    # sizes the matrix-core kernels take
+    (4, 2, 64, 16, [1, 1, 1, 1, 1], [1, 16, 17, 200, 1000], None),   # decodes: first token, page edges, long
+    (6, 2, 64, 16, [40, 1, 2, 100], [40, 77, 300, 100], None),       # three heads per kv head, mixed batch
+    (4, 1, 128, 32, [65, 1], [200, 31], None),                       # one kv head, pages of 32
+    (8, 2, 64, 16, [1, 1, 1], [50, 333, 64], 40),                    # decodes with a window
+    (8, 2, 64, 64, [130, 3, 1], [130, 250, 99], 33),                 # portions with a window, pages of 64
+    (16, 1, 64, 16, [1, 1], [129, 2], None),                         # sixteen heads on one kv head
+    (32, 1, 64, 16, [1, 70], [75, 70], None),                        # more heads per kv head than a wave's columns
 ]
 
 

@@ -89,7 +89,7 @@ def test_attention_part(dtype, window):
     S, first = 23, 14
     h = torch.randn(S, D, generator=gen(11)).to(dtype)
     cache = LayerCache(group=0, k=torch.zeros(16, nkv, page, hd, dtype=dtype, device=DEV),
-                       v=torch.zeros(16, nkv, page, hd, dtype=dtype, device=DEV), page_size=page)
+                       v=torch.zeros(16, nkv, hd, page, dtype=dtype, device=DEV), page_size=page)
     table = torch.tensor([[9, 2, 11, 5, 0, 7]], dtype=torch.int32, device=DEV)
     x = torch.zeros(S, D, device=DEV)
     for lo, hi in ((0, first), (first, S)):

@@ -36,7 +36,19 @@ TINY_C = dict(
 )
 TINY_C_INIT = dict(std=0.12, norm_init="uniform", block_size=16)
 
-ALL = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT)}
+# sizes the matrix-core kernels take (head_dim 64, pages of 16, widths in multiples of 8), so
+# that the bfloat16 engine runs them: 2 heads per kv head, llama3 scaling with a short context
+TINY_D = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=128, intermediate_size=272, num_hidden_layers=2,
+    num_attention_heads=4, num_key_value_heads=2, head_dim=64, vocab_size=520, max_position_embeddings=512,
+    rms_norm_eps=1e-5, rope_theta=50000.0,
+    rope_scaling=dict(rope_type="llama3", factor=4.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=128),
+    tie_word_embeddings=True,
+)
+TINY_D_INIT = dict(std=0.08, norm_init="uniform", block_size=16)
+
+ALL = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT), "D": (TINY_D, TINY_D_INIT)}
 
 
 def make_model_dir(tmp_path, name: str, seed: int = 0, storage: str = "bfloat16") -> str:
