@@ -1,0 +1,213 @@
+#!/usr/bin/python3
+"""Decode and prefill throughput of the engine on one MI355X (Llama 3.2 1B layer sizes).
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  ``value`` is decoded tokens per second at batch 8 with the context
+length of the benchmark configuration (every request's cache holds that many tokens when
+the timed steps end).  A "step" is one decode step of the whole batch through the engine's
+own path: metadata upload, the replayed graph (model + sampling kernel), and the copy of the
+chosen tokens back to the host, which the next step waits for.
+Also on the line: ``prefill`` (one 2,048-token prompt in one step), ``roofline`` (bytes the
+decode step has to read / its time, against 8 TB/s) and ``points`` (batch 1 and 64).
+Weights are random (N(0, 0.02), norms 1), token ids uniform random; no dataset is involved.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# layer sizes of Llama 3.2 1B (BASELINE.json configs[2])
+MODEL = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=8192, num_hidden_layers=16,
+    num_attention_heads=32, num_key_value_heads=8, head_dim=64, vocab_size=128256,
+    max_position_embeddings=131072, rms_norm_eps=1e-5, rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    tie_word_embeddings=True, torch_dtype="bfloat16",
+)
+CONTEXT = 4096
+PREFILL_TOKENS = 2048
+BLOCK_SIZE = 16
+HBM_PEAK_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def make_runner(cfg_raw, layers, dtype, max_batch, max_cache_tokens, seed=0):
+    import torch
+
+    from photon_infer_amd.engine import EngineOptions, ModelRunner
+    from photon_infer_amd.registry import build_model_spec, config_from_dict
+
+    raw = dict(cfg_raw, num_hidden_layers=layers)
+    cfg = config_from_dict(raw)
+    spec = build_model_spec(cfg)
+    tdtype = torch.bfloat16 if dtype == "bf16" else torch.float32
+    gen = torch.Generator(device="cuda").manual_seed(seed)
+    tensors = {}
+    for s in spec.tensor_specs():
+        if s.role == "norm":
+            tensors[s.name] = torch.ones(s.shape, dtype=tdtype, device="cuda")
+        else:
+            tensors[s.name] = (torch.randn(s.shape, generator=gen, device="cuda", dtype=torch.float32) * 0.02).to(tdtype)
+    opts = EngineOptions(dtype="bfloat16" if dtype == "bf16" else "float32", block_size=BLOCK_SIZE,
+                         max_cache_tokens=max_cache_tokens, max_batch=max_batch, max_model_len=CONTEXT + 64)
+    return ModelRunner(None, opts, config=cfg, tensors=tensors), cfg
+
+
+def weight_bytes(runner) -> int:
+    """Bytes of every tensor the decode step reads once (tied head counted once)."""
+    seen, total = set(), 0
+    m = runner.model
+    tensors = [m.head.weight, m.final_norm.weight]
+    for b in m.blocks:
+        tensors += [b.norm1.weight, b.norm2.weight, b.mixer.w_qkv, b.mixer.w_o, b.ffn.w_gate_up, b.ffn.w_down]
+    for t in tensors:
+        if t.data_ptr() not in seen:
+            seen.add(t.data_ptr())
+            total += t.numel() * t.element_size()
+    return total
+
+
+def kv_bytes_per_token(cfg, layers, elem) -> int:
+    return 2 * layers * cfg.num_key_value_heads * cfg.head_dim * elem
+
+
+def prefill_flops(cfg, layers, T) -> float:
+    per_layer = cfg.hidden_size * (cfg.q_size + 2 * cfg.kv_size) + cfg.q_size * cfg.hidden_size \
+        + 3 * cfg.hidden_size * cfg.intermediate_size
+    gemm = 2.0 * T * per_layer * layers
+    attn = layers * 2 * 2.0 * cfg.num_attention_heads * cfg.head_dim * (T * (T + 1) / 2)
+    head = 2.0 * cfg.hidden_size * cfg.vocab_size
+    return gemm + attn + head
+
+
+def time_decode(runner, batch, steps, warmup, context, seed=1):
+    """Median-free, plain timing: ``steps`` decode steps of ``batch`` requests that end at ``context``."""
+    import torch
+
+    from photon_infer_amd.engine import StepEntry
+
+    vocab = runner.spec.vocab_size
+    g = torch.Generator().manual_seed(seed)
+    start_len = context - steps - warmup
+    assert start_len >= 1
+    rids = [f"d{batch}_{i}" for i in range(batch)]
+    for rid in rids:
+        runner.admit(rid)
+        toks = torch.randint(0, vocab, (start_len,), generator=g).tolist()
+        for i in range(0, start_len, 2048):
+            runner.step([StepEntry(rid, toks[i:i + 2048])])
+    last = torch.randint(0, vocab, (batch,), generator=g).tolist()
+    temps, draws = [0.0] * batch, [0.0] * batch
+
+    def one_step(tokens):
+        out = runner.decode_step([StepEntry(rid, [t], [0]) for rid, t in zip(rids, tokens)], temps, draws)
+        return out.tolist()       # the next step needs these: the copy back is part of the step
+
+    for _ in range(warmup):
+        last = one_step(last)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        last = one_step(last)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    mean_ctx = context - (steps - 1) / 2.0        # keys each request reads, averaged over the timed steps
+    for rid in rids:
+        runner.release(rid)
+    return dt / steps, mean_ctx
+
+
+def time_prefill(runner, tokens, reps, seed=2):
+    import torch
+
+    from photon_infer_amd.engine import StepEntry
+
+    g = torch.Generator().manual_seed(seed)
+    toks = torch.randint(0, runner.spec.vocab_size, (tokens,), generator=g).tolist()
+
+    def once(i):
+        rid = f"p{i}"
+        runner.admit(rid)
+        logits = runner.step([StepEntry(rid, toks, [tokens - 1])])
+        runner.release(rid)
+        return logits
+
+    once(-1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(reps):
+        once(i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / reps
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"],
+                    help="fewer layers than the model has, if memory or time needs it (both numbers are reported)")
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU available", file=sys.stderr)
+        return 1
+    elem = 2 if args.dtype == "bf16" else 4
+    big = 1 if args.no_points else 64
+    runner, cfg = make_runner(MODEL, args.layers, args.dtype, max(big, args.batch), (max(big, args.batch)) * (CONTEXT + 64))
+    wbytes = weight_bytes(runner)
+    kvb = kv_bytes_per_token(cfg, args.layers, elem)
+
+    sec, mean_ctx = time_decode(runner, args.batch, args.steps, args.warmup, CONTEXT)
+    value = args.batch / sec
+    step_bytes = wbytes + args.batch * mean_ctx * kvb
+    achieved = step_bytes / sec / 1e9
+    line = {
+        "metric": "decode tok/s at batch 8, context 4096 (Llama 3.2 1B layer sizes, random weights)",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+        "config": {
+            "model": "llama-3.2-1b-sizes", "layers": args.layers, "layers_of_model": MODEL["num_hidden_layers"],
+            "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+            "tied_embeddings": cfg.tie_word_embeddings, "rope": "llama3 theta=500000 factor=32",
+            "global_batch": args.batch, "seq_len": CONTEXT, "kv_block": BLOCK_SIZE, "prefill_tokens": PREFILL_TOKENS,
+            "parallelism": "single-gpu", "weight_bytes": wbytes, "kv_bytes_per_token": kvb,
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_points:
+        psec = time_prefill(runner, PREFILL_TOKENS, 5)
+        flops = prefill_flops(cfg, args.layers, PREFILL_TOKENS)
+        line["prefill"] = {"value": round(PREFILL_TOKENS / psec, 1), "tokens": PREFILL_TOKENS, "ms": round(psec * 1e3, 3),
+                           "frac": round(flops / psec / PEAK_FLOPS[args.dtype], 4)}
+        points = {}
+        for b in (1, 64):
+            s, _ = time_decode(runner, b, args.steps, args.warmup, CONTEXT)
+            points[f"decode_b{b}"] = round(b / s, 1)
+        line["points"] = points
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

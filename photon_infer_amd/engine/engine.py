@@ -82,13 +82,17 @@ class ContinuousBatchEngine:
             entries.append(StepEntry(req.request_id, req.next_tokens(n), [n - 1] if ends else []))
             if ends:
                 sampled_reqs.append(req)
-        logits = self.runner.step(entries)
+        temps = [r.params.temperature for r in sampled_reqs]
+        draws = [uniform_draw(r.params.seed, r.num_generated()) if r.params.temperature > 0 else 0.0
+                 for r in sampled_reqs]
         tokens: List[int] = []
-        if sampled_reqs:
-            temps = [r.params.temperature for r in sampled_reqs]
-            draws = [uniform_draw(r.params.seed, r.num_generated()) if r.params.temperature > 0 else 0.0
-                     for r in sampled_reqs]
-            tokens = self.sampler.sample(logits, temps, draws)
+        if self.options.use_graphs and len(sampled_reqs) == len(entries) and all(n == 1 for _, n in batch.items):
+            # single tokens only, every one sampled: the replayed graph (model + sampling kernel)
+            tokens = self.runner.decode_step(entries, temps, draws).tolist()
+        else:
+            logits = self.runner.step(entries)
+            if sampled_reqs:
+                tokens = self.sampler.sample(logits, temps, draws)
         done = []
         for req, n in batch.items:
             req.add_computed_tokens(n)

@@ -20,7 +20,7 @@ import torch
 
 from .. import ops
 from ..cache import CacheManager, StateSlots
-from ..errors import CacheError, RequestError
+from ..errors import CacheError, OutOfPagesError, RequestError
 from ..parts import DecoderModel, LayerCache, ModelSpec, StepContext, plan_cache
 from ..registry import build_model_spec, load_config
 from ..weights import load_model_tensors
@@ -39,20 +39,29 @@ class StepEntry:
 class ModelRunner:
     """Owns the model, the cache (manager + device pools + state slabs) and ``step``."""
 
-    def __init__(self, model_dir: str, options: Optional[EngineOptions] = None):
+    def __init__(self, model_dir: Optional[str], options: Optional[EngineOptions] = None, *, config=None,
+                 tensors: Optional[Dict[str, torch.Tensor]] = None):
+        """From a model folder, or (``model_dir`` None) from a typed config and tensors that are
+        already on the device, named and shaped as the model's tensor list says."""
         self.options = options or EngineOptions()
         self.dtype = self.options.resolved_dtype()
         self.device = torch.device(self.options.device)
         if self.device.type != "cuda" or not torch.cuda.is_available():
             raise RequestError("the engine runs on a GPU only; no CUDA/HIP device is available")
         ops.ensure_loaded(self.dtype)
-        self.config = load_config(model_dir)
+        self.config = load_config(model_dir) if model_dir is not None else config
         self.spec: ModelSpec = build_model_spec(self.config)
-        tensors = load_model_tensors(model_dir, self.spec.tensor_specs(), self.dtype, self.device, self.spec.ignorable)
+        if model_dir is not None:
+            tensors = load_model_tensors(model_dir, self.spec.tensor_specs(), self.dtype, self.device, self.spec.ignorable)
+        else:
+            from ..weights.loader import check_tensors
+            check_tensors({t.name: t for t in self.spec.tensor_specs()}, {n: tuple(t.shape) for n, t in tensors.items()},
+                          self.spec.ignorable, "given tensors")
         self.model = DecoderModel(self.spec)
         self.model.load(tensors, self.dtype, self.device)
         del tensors
         self._build_cache()
+        self._graphs: Dict[int, "_DecodeGraph"] = {}
 
     # ------------------------------------------------------------------ cache set-up
     def _build_cache(self) -> None:
@@ -108,8 +117,9 @@ class ModelRunner:
             n = len(e.tokens)
             if n == 0:
                 raise RequestError(f"request {e.rid!r} brings no tokens")
-            bad = [t for t in e.tokens if not 0 <= int(t) < vocab]
-            if bad:
+            arr = np.asarray(e.tokens)
+            if arr.dtype.kind not in "iu" or arr.min() < 0 or arr.max() >= vocab:
+                bad = [t for t in e.tokens if not (isinstance(t, (int, np.integer)) and 0 <= int(t) < vocab)]
                 raise RequestError(f"request {e.rid!r}: token id {bad[0]} is outside the vocabulary of {vocab}")
             for w in e.want:
                 if not 0 <= int(w) < n:
@@ -155,6 +165,19 @@ class ModelRunner:
         ops.attach_attention_plan(ctx, extra, views)
         return ctx
 
+    def _reserve(self, entries: Sequence[StepEntry]) -> None:
+        """Pages for the step's new tokens: refuse the whole step before taking any page."""
+        held = [0] * len(self.cache.groups)
+        for e in entries:
+            need = self.cache.pages_needed(e.rid, len(e.tokens))
+            held = [h + n for h, n in zip(held, need)]
+        for g, h in enumerate(held):
+            if h > self.cache.free_pages(g):
+                raise OutOfPagesError(
+                    f"the step needs {h} more pages in cache group {g}, {self.cache.free_pages(g)} are free")
+        for e in entries:
+            self.cache.reserve(e.rid, len(e.tokens))
+
     @torch.no_grad()
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits [wanted rows, vocab] on the device, in
@@ -163,23 +186,31 @@ class ModelRunner:
         if not entries:
             return None
         self._check(entries)
-        # pages for the new tokens: refuse the whole step before taking any page
-        held = [0] * len(self.cache.groups)
-        for e in entries:
-            need = self.cache.pages_needed(e.rid, len(e.tokens))
-            held = [h + n for h, n in zip(held, need)]
-        for g, h in enumerate(held):
-            if h > self.cache.free_pages(g):
-                from ..errors import OutOfPagesError
-                raise OutOfPagesError(
-                    f"the step needs {h} more pages in cache group {g}, {self.cache.free_pages(g)} are free")
-        for e in entries:
-            self.cache.reserve(e.rid, len(e.tokens))
+        self._reserve(entries)
         ctx = self.build_context(entries)
         logits = self.model.forward(ctx, self.layer_caches)
         for e in entries:
             self.cache.commit(e.rid, len(e.tokens))
         return logits
+
+    @torch.no_grad()
+    def decode_step(self, entries: Sequence[StepEntry], temperatures: Sequence[float],
+                    uniforms: Sequence[float]) -> torch.Tensor:
+        """A batch of single tokens, one per request, each wanting its next token: the model
+        and the sampling kernel run as one replayed HIP graph (captured per batch size at
+        first use).  Returns the chosen token ids (int32 [R], on the device)."""
+        entries = list(entries)
+        self._check(entries)
+        if any(len(e.tokens) != 1 for e in entries):
+            raise RequestError("decode_step takes exactly one token per request")
+        self._reserve(entries)
+        graph = self._graphs.get(len(entries))
+        if graph is None:
+            graph = self._graphs[len(entries)] = _DecodeGraph(self, len(entries))
+        out = graph.run(entries, temperatures, uniforms)
+        for e in entries:
+            self.cache.commit(e.rid, 1)
+        return out
 
 
 def _upload(parts: Dict[str, np.ndarray], device) -> Dict[str, torch.Tensor]:
@@ -194,3 +225,81 @@ def _upload(parts: Dict[str, np.ndarray], device) -> Dict[str, torch.Tensor]:
         packed[o:o + n] = arr
     dev = torch.from_numpy(packed).to(device)
     return {name: dev[o:o + n] for name, (o, n) in offsets.items()}
+
+
+class _DecodeGraph:
+    """The decode step of one batch size as a HIP graph.
+
+    All metadata lives in one device buffer at fixed addresses (tokens, positions, lengths,
+    slots, sampling parameters, block-table rows of full width); a step copies the new values
+    in and replays.  Nothing in the graph depends on a host-side number: the attention grid is
+    fixed by the batch size, key ranges are derived on the device from the lengths.
+    """
+
+    def __init__(self, runner: "ModelRunner", R: int):
+        self.runner, self.R = runner, R
+        cache = runner.cache
+        self.width = cache.max_blocks
+        G = len(cache.groups)
+        names = ["token_ids", "positions", "req_of_token", "kv_len", "slots", "logit_rows", "temps", "uniforms"]
+        self.off, total = {}, 0
+        for name in names:
+            self.off[name] = (total, R)
+            total += (R + 3) // 4 * 4
+        self.off["q_start"] = (total, R + 1)
+        total += (R + 1 + 3) // 4 * 4
+        for g in range(G):
+            self.off[f"table{g}"] = (total, R * self.width)
+            total += (R * self.width + 3) // 4 * 4
+        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.h = {k: self.host[o:o + n].numpy() for k, (o, n) in self.off.items()}
+        self.hf = {k: self.host[o:o + n].view(torch.float32).numpy() for k, (o, n) in self.off.items() if k in ("temps", "uniforms")}
+        self.h["req_of_token"][:] = np.arange(R)
+        self.h["logit_rows"][:] = np.arange(R)
+        self.h["q_start"][:] = np.arange(R + 1)
+        self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
+        d = {k: self.dev[o:o + n] for k, (o, n) in self.off.items()}
+        self.ctx = StepContext(
+            T=R, R=R, dtype=runner.dtype, token_ids=d["token_ids"], positions=d["positions"],
+            req_of_token=d["req_of_token"], q_start=d["q_start"], kv_len=d["kv_len"], slots=d["slots"],
+            block_tables={g: d[f"table{g}"].view(R, self.width) for g in range(G)}, logit_rows=d["logit_rows"],
+            q_lens=[1] * R, kv_lens=(), max_q_len=1, max_kv_len=None, all_decode=True)
+        self.ctx.decode_splits_fixed = True       # key ranges by batch size only, not by the lengths of the day
+        self.temps = d["temps"].view(torch.float32)
+        self.uniforms = d["uniforms"].view(torch.float32)
+        self.sampled = torch.zeros(R, dtype=torch.int32, device=runner.device)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+
+    def _fill(self, entries, temperatures, uniforms) -> None:
+        cache = self.runner.cache
+        slots = [cache.slot(e.rid) for e in entries]
+        lengths = np.fromiter((cache.length(e.rid) for e in entries), np.int32, self.R)
+        self.h["token_ids"][:] = [e.tokens[0] for e in entries]
+        self.h["positions"][:] = lengths
+        self.h["kv_len"][:] = lengths + 1
+        self.h["slots"][:] = slots
+        self.hf["temps"][:] = temperatures
+        self.hf["uniforms"][:] = uniforms
+        for g in range(len(cache.groups)):
+            self.h[f"table{g}"].reshape(self.R, self.width)[:] = cache.table_rows(g, slots, self.width)
+        self.ctx.host_slots = slots
+        self.dev.copy_(self.host, non_blocking=True)
+
+    def _body(self) -> None:
+        logits = self.runner.model.forward(self.ctx, self.runner.layer_caches)
+        ops.sample(self.sampled, logits, self.temps, self.uniforms)
+
+    def run(self, entries, temperatures, uniforms) -> torch.Tensor:
+        self._fill(entries, temperatures, uniforms)
+        if self.graph is None:
+            # the first step of this batch size runs eagerly (and does this step's work); the
+            # capture that follows records the same launches without running them
+            self._body()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                self._body()
+            self.graph = graph
+        else:
+            self.graph.replay()
+        return self.sampled

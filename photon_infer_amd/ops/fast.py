@@ -146,7 +146,8 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
     G = num_heads // num_kv_heads
     R = ctx.R
     if ctx.all_decode and G <= 16:
-        splits = getattr(ctx, "decode_splits_fixed", None) or decode_splits(R, num_kv_heads, ctx.max_kv_len)
+        fixed = getattr(ctx, "decode_splits_fixed", False)
+        splits = decode_splits(R, num_kv_heads, None if fixed else ctx.max_kv_len)
         ws = workspace(q.device)
         while splits > 1 and R * num_heads * splits * (head_dim + 4) > ws.attn_part.numel():
             splits -= 1

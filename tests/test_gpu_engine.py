@@ -138,3 +138,29 @@ def test_command_line(model_dirs, tmp_path):
         capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stderr[-2000:]
     assert "User: hi there" in proc.stdout and "Prompt tokens: 9" in proc.stdout and "Assistant:" in proc.stdout
+
+
+@pytest.mark.parametrize("dtype,name", [("float32", "A"), ("bfloat16", "D")])
+def test_graph_replayed_decode_equals_eager_steps(tmp_path, dtype, name):
+    """Decode-only steps replay a captured graph (model + sampling kernel); every replay must
+    give what the eager step gives, with eager work (new requests' prompts) between replays."""
+    d = make_model_dir(tmp_path, name, seed=31)
+    vocab = ALL[name][0]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 90 + n) for n in (3, 40, 17, 9)]
+
+    def run(use_graphs):
+        eng = engine(d, name, dtype=dtype, use_graphs=use_graphs, chunk_size=8, max_step_tokens=24)
+        ids = [eng.add_request(p, 14 + 3 * i, temperature=0.7 if i % 2 else 0.0, seed=7 + i, ignore_eos=True)
+               for i, p in enumerate(prompts[:3])]
+        for _ in range(12):
+            eng.step()
+        ids.append(eng.add_request(prompts[3], 9, ignore_eos=True))     # arrives mid-run: eager steps between replays
+        eng.run_until_complete()
+        return [eng.get_result(i) for i in ids], eng
+
+    eager, _ = run(False)
+    graphed, eng = run(True)
+    assert eng.runner._graphs, "no decode step went through a graph"
+    assert all(g.graph is not None for g in eng.runner._graphs.values())
+    assert graphed == eager
+    assert [len(x) for x in graphed] == [14, 17, 20, 9]
