@@ -38,17 +38,31 @@ extern "C" int pi_embedding(float* out, const void* table, int table_dtype, cons
 // ------------------------------------------------------------------ RMS norm
 // y[m, :] = w * (x[r, :] * (1 / sqrt(mean(x[r, :]^2) + eps))), r = rows ? rows[m] : m.
 // Sum of squares, root and scaling in float32; one rounding on store.
+// With `part` (float32 [splits, x_rows, D]: the pieces of a matrix product that is still to be
+// added to x), row r first becomes x[r, :] + sum_s part[s, r, :] (in split order), is written
+// back to x, and is then normalised: the residual add, the split reduction and the norm in one pass.
 template <typename TO, typename TW>
-__global__ void rmsnorm_kernel(TO* __restrict__ out, const float* __restrict__ x, const int* __restrict__ rows,
-                               const TW* __restrict__ w, float eps, int D) {
+__global__ void rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ x, const int* __restrict__ rows,
+                               const TW* __restrict__ w, float eps, int D, const float* __restrict__ part, int splits,
+                               long part_stride) {
   __shared__ float scratch[16];
   const long m = blockIdx.x;
   const long r = rows ? rows[m] : m;
-  const float* xr = x + r * D;
+  float* xr = x + r * D;
   float ss = 0.f;
-  for (int i = threadIdx.x; i < D; i += blockDim.x) {
-    const float v = xr[i];
-    ss += v * v;
+  if (part) {
+    const float* pr = part + r * D;
+    for (int i = threadIdx.x; i < D; i += blockDim.x) {
+      float v = xr[i];
+      for (int s = 0; s < splits; ++s) v += pr[s * part_stride + i];
+      xr[i] = v;               // the same thread reads it back below
+      ss += v * v;
+    }
+  } else {
+    for (int i = threadIdx.x; i < D; i += blockDim.x) {
+      const float v = xr[i];
+      ss += v * v;
+    }
   }
   ss = block_sum(ss, scratch);
   const float inv = 1.0f / sqrtf(ss / (float)D + eps);
@@ -56,13 +70,16 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, const float* __restrict__ x
   for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = from_float<TO>(to_float(w[i]) * (xr[i] * inv));
 }
 
-extern "C" int pi_rmsnorm(void* out, int out_dtype, const float* x, const int* rows, const void* w, int w_dtype,
-                          float eps, int M, int D, hipStream_t stream) {
+// part == nullptr: plain norm.  Otherwise part is float32 [splits, x_rows, D].
+extern "C" int pi_rmsnorm(void* out, int out_dtype, float* x, const int* rows, const void* w, int w_dtype, float eps, int M,
+                          int D, const float* part, int splits, long x_rows, hipStream_t stream) {
   PI_REQUIRE(M >= 0 && D > 0, "rmsnorm: bad sizes M=%d D=%d", M, D);
+  PI_REQUIRE(part == nullptr || (splits >= 1 && x_rows > 0), "rmsnorm: bad split description (%d splits, %ld rows)", splits, x_rows);
   if (M == 0) return 0;
   const int threads = D >= 1024 ? 256 : (D >= 256 ? 128 : 64);
+  const long stride = x_rows * (long)D;
 #define LAUNCH(TO, TW) \
-  hipLaunchKernelGGL((rmsnorm_kernel<TO, TW>), dim3(M), dim3(threads), 0, stream, (TO*)out, x, rows, (const TW*)w, eps, D)
+  hipLaunchKernelGGL((rmsnorm_kernel<TO, TW>), dim3(M), dim3(threads), 0, stream, (TO*)out, x, rows, (const TW*)w, eps, D, part, splits, stride)
   if (out_dtype == PI_F32 && w_dtype == PI_F32) LAUNCH(float, float);
   else if (out_dtype == PI_F32 && w_dtype == PI_BF16) LAUNCH(float, bf16_t);
   else if (out_dtype == PI_BF16 && w_dtype == PI_F32) LAUNCH(bf16_t, float);
@@ -115,6 +132,10 @@ extern "C" int pi_swiglu(void* out, const void* gu, int dtype, int T, int I, int
 // fixed feature - the order in which the matrix-core attention kernels contract them.
 // angle = float(pos) * inv_freq[j]; pair j is (x[j], x[j + R/2]) or, interleaved,
 // (x[2j], x[2j+1]); (a, b) <- (a cos - b sin, a sin + b cos).  Dims >= R are copied.
+// The source of q, k, v is either the projection's output in the compute dtype (q is rotated in
+// place) or, when `part` is given, the pieces of that projection still to be summed: float32
+// [splits, T, ncols] with q at column q_col, k at k_col, v at v_col; the rotated q then goes to
+// the q buffer, and nothing ever holds the unrotated values in reduced precision.
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
                                      const T* __restrict__ v, long v_stride, const int* __restrict__ positions,
@@ -122,17 +143,22 @@ __global__ void rope_kv_write_kernel(T* __restrict__ q, long q_stride, const T* 
                                      int rotary_dim, int interleaved, int nh, int nkv_write, int nkv, int hd,
                                      T* __restrict__ k_cache, T* __restrict__ v_cache,
                                      const int* __restrict__ block_table, int table_width, int page_size,
-                                     long num_pages) {
+                                     long num_pages, const float* __restrict__ part, int splits, long part_stride,
+                                     int ncols, int q_col, int k_col, int v_col) {
+  __shared__ float head[256];
   const long t = blockIdx.x;
   const int h = blockIdx.y;
   const int lane = threadIdx.x;
   const int pos = positions[t];
-  const T* src;
   T* dst;
+  long dst_stride = 1;        // element stride of the destination (values are stored transposed)
+  const T* src = nullptr;
+  int col = 0;
   bool rotate = rotary_dim > 0;
   if (h < nh) {
     dst = q + t * q_stride + (long)h * hd;
     src = dst;
+    col = q_col + h * hd;
   } else {
     const int hh = h - nh;
     const bool is_v = hh >= nkv_write;
@@ -142,34 +168,46 @@ __global__ void rope_kv_write_kernel(T* __restrict__ q, long q_stride, const T* 
     if (blk >= table_width) return;
     const long page = block_table[(long)r * table_width + blk];
     if (page < 0 || page >= num_pages) return;  // the host checks tables; never write outside the pool
-    const long off = ((page * nkv + g) * page_size + (pos % page_size)) * hd;
     if (is_v) {
-      const T* vs = v + t * v_stride + (long)g * hd;
-      T* vd = v_cache + (page * nkv + g) * (long)page_size * hd + (pos % page_size);
-      for (int d = lane; d < hd; d += PI_WAVE) vd[(long)d * page_size] = vs[d];
-      return;
+      src = v ? v + t * v_stride + (long)g * hd : nullptr;
+      col = v_col + g * hd;
+      dst = v_cache + (page * nkv + g) * (long)page_size * hd + (pos % page_size);
+      dst_stride = page_size;
+      rotate = false;
     } else {
-      src = k + t * k_stride + (long)g * hd;
-      dst = k_cache + off;
+      src = k ? k + t * k_stride + (long)g * hd : nullptr;
+      col = k_col + g * hd;
+      dst = k_cache + ((page * nkv + g) * page_size + (pos % page_size)) * hd;
     }
   }
+  // the head's values in float32
+  for (int d = lane; d < hd; d += PI_WAVE) {
+    float val;
+    if (part) {
+      val = 0.f;
+      const float* p = part + t * ncols + col + d;
+      for (int s = 0; s < splits; ++s) val += p[s * part_stride];
+    } else {
+      val = to_float(src[d]);
+    }
+    head[d] = val;
+  }
+  __syncthreads();
   if (rotate) {
     const int half = rotary_dim / 2;
     for (int j = lane; j < half; j += PI_WAVE) {
       const int i0 = interleaved ? 2 * j : j;
       const int i1 = interleaved ? 2 * j + 1 : j + half;
-      const float a = to_float(src[i0]);
-      const float b = to_float(src[i1]);
+      const float a = head[i0], b = head[i1];
       const float angle = (float)pos * inv_freq[j];
       float s, c;
       sincosf(angle, &s, &c);
-      dst[i0] = from_float<T>(a * c - b * s);
-      dst[i1] = from_float<T>(a * s + b * c);
+      dst[i0 * dst_stride] = from_float<T>(a * c - b * s);
+      dst[i1 * dst_stride] = from_float<T>(a * s + b * c);
     }
-    if (dst != src)
-      for (int i = rotary_dim + lane; i < hd; i += PI_WAVE) dst[i] = src[i];
-  } else if (dst != src) {
-    for (int i = lane; i < hd; i += PI_WAVE) dst[i] = src[i];
+    for (int i = rotary_dim + lane; i < hd; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(head[i]);
+  } else {
+    for (int i = lane; i < hd; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(head[i]);
   }
 }
 
@@ -177,12 +215,14 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
                                 int dtype, const int* positions, const int* req_of_token, const float* inv_freq,
                                 int rotary_dim, int interleaved, int T, int nh, int nkv, int hd, int write_kv,
                                 void* k_cache, void* v_cache, const int* block_table, int table_width,
-                                int page_size, long num_pages, hipStream_t stream) {
-  PI_REQUIRE(T >= 0 && nh >= 0 && nkv >= 0 && hd > 0, "rope_kv_write: bad sizes T=%d heads=%d kv_heads=%d head_dim=%d", T, nh, nkv, hd);
+                                int page_size, long num_pages, const float* part, int splits, int ncols, int q_col,
+                                int k_col, int v_col, hipStream_t stream) {
+  PI_REQUIRE(T >= 0 && nh >= 0 && nkv >= 0 && hd > 0 && hd <= 256, "rope_kv_write: bad sizes T=%d heads=%d kv_heads=%d head_dim=%d", T, nh, nkv, hd);
   PI_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && rotary_dim % 2 == 0, "rope_kv_write: rotary_dim %d must be even and <= head_dim %d", rotary_dim, hd);
   PI_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "rope_kv_write: rotation asked for without a frequency table");
+  PI_REQUIRE(part == nullptr || (splits >= 1 && ncols > 0), "rope_kv_write: bad split description");
   if (write_kv) {
-    PI_REQUIRE(k && v && k_cache && v_cache && block_table && req_of_token, "rope_kv_write: cache write asked for without k/v/cache/table");
+    PI_REQUIRE((part || (k && v)) && k_cache && v_cache && block_table && req_of_token, "rope_kv_write: cache write asked for without k/v/cache/table");
     PI_REQUIRE(page_size > 0 && table_width > 0 && num_pages > 0, "rope_kv_write: bad cache geometry page_size=%d table_width=%d pages=%ld", page_size, table_width, num_pages);
   }
   const int heads = nh + (write_kv ? 2 * nkv : 0);
@@ -190,14 +230,17 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
   PI_REQUIRE(heads <= 65535, "rope_kv_write: too many heads (%d)", heads);
   const dim3 grid(T, heads), block(PI_WAVE);
   const int nkv_write = write_kv ? nkv : 0;
+  const long part_stride = (long)T * ncols;
   if (dtype == PI_F32)
     hipLaunchKernelGGL(rope_kv_write_kernel<float>, grid, block, 0, stream, (float*)q, q_stride, (const float*)k, k_stride,
                        (const float*)v, v_stride, positions, req_of_token, inv_freq, rotary_dim, interleaved, nh, nkv_write,
-                       nkv, hd, (float*)k_cache, (float*)v_cache, block_table, table_width, page_size, num_pages);
+                       nkv, hd, (float*)k_cache, (float*)v_cache, block_table, table_width, page_size, num_pages, part,
+                       splits, part_stride, ncols, q_col, k_col, v_col);
   else if (dtype == PI_BF16)
     hipLaunchKernelGGL(rope_kv_write_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)q, q_stride, (const bf16_t*)k, k_stride,
                        (const bf16_t*)v, v_stride, positions, req_of_token, inv_freq, rotary_dim, interleaved, nh, nkv_write,
-                       nkv, hd, (bf16_t*)k_cache, (bf16_t*)v_cache, block_table, table_width, page_size, num_pages);
+                       nkv, hd, (bf16_t*)k_cache, (bf16_t*)v_cache, block_table, table_width, page_size, num_pages, part,
+                       splits, part_stride, ncols, q_col, k_col, v_col);
   else
     return pi_fail("rope_kv_write: unsupported dtype %d", dtype);
   return pi_check_launch("rope_kv_write");

@@ -7,8 +7,8 @@
 // cover 128 contiguous bytes.  No LDS on the way in: activations come from L2.
 // A block is four waves on the same 32 rows, each on a quarter of the block's k-range; they
 // add up through LDS.  The k-range may further be split over blocks (grid.y): each block
-// writes its partial tile, and the block that arrives last at the tile's counter adds the
-// partials in split order (deterministic) and applies the epilogue.  Counters reset themselves.
+// then writes its partial tile to a workspace and the consumer of the product adds the
+// partials in split order (deterministic).
 //
 // Epilogues as in the many-row kernel: store bf16, store f32, add into f32, SwiGLU (gate / up
 // rows interleaved by 16, so the two row tiles of a wave are the gate and the up rows of the
@@ -30,10 +30,8 @@ __device__ inline void epilogue_store(void* Cv, long ldc, long m, long n, float 
 template <int MB, int EPI>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ X, long ldx,
                                                           const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
-                                                          int k_per_block, float* __restrict__ part,
-                                                          int* __restrict__ counters) {
+                                                          int k_per_block, float* __restrict__ part) {
   __shared__ float red[4][ROWS_PER_BLOCK][MB * 16 + 1];
-  __shared__ int is_last;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int lr = lane % 16, lg = lane / 16;
   const long n0 = (long)blockIdx.x * ROWS_PER_BLOCK;
@@ -128,33 +126,46 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
     return;
   }
 
-  // k split over blocks: publish this block's partial tile, the last arrival finishes the tile
+  // k split over blocks: this block's partial tile goes to part[split][m][n]; whoever consumes
+  // the product (the reduce kernel below, or a norm / rotation kernel that folds the sum into
+  // its own read) adds the splits in split order.  No block waits for or signals another:
+  // on a chip of several dies a device-wide fence costs more than a kernel boundary.
   float* mine = part + (long)blockIdx.y * M * N;
   for (int idx = tid; idx < ROWS_PER_BLOCK * cols; idx += 256) {
     const int nl = idx % ROWS_PER_BLOCK, m = idx / ROWS_PER_BLOCK;
     if (m >= M || n0 + nl >= N) continue;
     mine[(long)m * N + n0 + nl] = red[0][nl][m] + red[1][nl][m] + red[2][nl][m] + red[3][nl][m];
   }
-  __threadfence();
-  __syncthreads();
-  if (tid == 0) is_last = (atomicAdd(&counters[blockIdx.x], 1) == splits - 1);
-  __syncthreads();
-  if (!is_last) return;
-  __threadfence();
-  for (int idx = tid; idx < ROWS_PER_BLOCK * cols; idx += 256) {
-    const int nl = idx % ROWS_PER_BLOCK, m = idx / ROWS_PER_BLOCK;
-    if (m >= M || n0 + nl >= N) continue;
-    float sum = 0.f;
-    for (int s = 0; s < splits; ++s) sum += __builtin_nontemporal_load(part + ((long)s * M + m) * N + n0 + nl);
-    epilogue_store<EPI>(Cv, ldc, m, n0 + nl, sum);
+}
+
+// C[m][n] (op)= sum over splits of part[s][m][n], in split order.
+template <int EPI>
+__global__ void splitk_reduce_kernel(void* __restrict__ Cv, long ldc, const float* __restrict__ part, int splits, int M, int N) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)M * N) return;
+  const long m = idx / N, n = idx % N;
+  float sum = 0.f;
+  for (int s = 0; s < splits; ++s) sum += part[(long)s * M * N + idx];
+  epilogue_store<EPI>(Cv, ldc, m, n, sum);
+}
+
+extern "C" int pi_splitk_reduce(void* C, int epilogue, long ldc, const void* part, int splits, int M, int N, hipStream_t stream) {
+  PI_REQUIRE(M > 0 && N > 0 && splits >= 1 && part, "splitk_reduce: bad arguments M=%d N=%d splits=%d", M, N, splits);
+  const long total = (long)M * N;
+  const dim3 grid((unsigned)((total + 255) / 256)), block(256);
+  switch (epilogue) {
+    case EPI_BF16: hipLaunchKernelGGL(splitk_reduce_kernel<EPI_BF16>, grid, block, 0, stream, C, ldc, (const float*)part, splits, M, N); break;
+    case EPI_F32: hipLaunchKernelGGL(splitk_reduce_kernel<EPI_F32>, grid, block, 0, stream, C, ldc, (const float*)part, splits, M, N); break;
+    case EPI_ACCUM: hipLaunchKernelGGL(splitk_reduce_kernel<EPI_ACCUM>, grid, block, 0, stream, C, ldc, (const float*)part, splits, M, N); break;
+    default: return pi_fail("splitk_reduce: unknown epilogue %d", epilogue);
   }
-  if (tid == 0) counters[blockIdx.x] = 0;
+  return pi_check_launch("splitk_reduce");
 }
 
 template <int MB>
 static int launch_mb(int epi, dim3 grid, hipStream_t stream, void* C, long ldc, const bf16_t* X, long ldx, const bf16_t* W,
-                     long ldw, int M, int N, int K, int kpb, float* part, int* counters) {
-#define GO(E) hipLaunchKernelGGL((gemm_skinny_kernel<MB, E>), grid, dim3(256), 0, stream, C, ldc, X, ldx, W, ldw, M, N, K, kpb, part, counters)
+                     long ldw, int M, int N, int K, int kpb, float* part) {
+#define GO(E) hipLaunchKernelGGL((gemm_skinny_kernel<MB, E>), grid, dim3(256), 0, stream, C, ldc, X, ldx, W, ldw, M, N, K, kpb, part)
   switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
     case EPI_F32: GO(EPI_F32); break;
@@ -166,31 +177,29 @@ static int launch_mb(int epi, dim3 grid, hipStream_t stream, void* C, long ldc, 
   return pi_check_launch("gemm_skinny");
 }
 
-// splits > 1 needs `part` (float32 [splits, M, N]) and `counters` (int32 [ceil(N / 32)], zero).
+// splits > 1: the partial products go to `part` (float32 [splits, M, N]) and C is not touched;
+// *splits_out tells how many splits were made (no empty ones).
 extern "C" int pi_gemm_skinny(void* C, int epilogue, long ldc, const void* X, long ldx, const void* W, long ldw, int M,
-                              int N, int K, int splits, void* part, long part_elems, void* counters, long num_counters,
-                              hipStream_t stream) {
+                              int N, int K, int splits, void* part, long part_elems, int* splits_out, hipStream_t stream) {
   PI_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: takes 1..64 rows, got M=%d N=%d K=%d", M, N, K);
   PI_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "gemm_skinny: K (%d) and row strides (%ld, %ld) must be multiples of 8", K, ldx, ldw);
   PI_REQUIRE(((uintptr_t)X % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_skinny: operands must be 16-byte aligned");
   PI_REQUIRE(splits >= 1 && splits <= 65535, "gemm_skinny: bad split count %d", splits);
   PI_REQUIRE(epilogue != EPI_SWIGLU || (splits == 1 && N % 32 == 0), "gemm_skinny: the SwiGLU epilogue needs one split and N (%d) a multiple of 32", N);
   const int groups = ceil_div(N, ROWS_PER_BLOCK);
-  if (splits > 1) {
-    PI_REQUIRE(part && counters, "gemm_skinny: a k-split needs a workspace");
-    PI_REQUIRE(part_elems >= (long)splits * M * N && num_counters >= groups, "gemm_skinny: workspace too small (%ld floats for %ld, %ld counters for %d)",
-               part_elems, (long)splits * M * N, num_counters, groups);
-  }
   int kpb = ceil_div(K, splits);
   kpb = ((kpb + KSTEP - 1) / KSTEP) * KSTEP;
   splits = ceil_div(K, kpb);                      // no empty splits
+  if (splits > 1)
+    PI_REQUIRE(part && part_elems >= (long)splits * M * N, "gemm_skinny: workspace too small (%ld floats for %ld)", part_elems, (long)splits * M * N);
+  if (splits_out) *splits_out = splits;
   const dim3 grid(groups, splits);
   const int mb = (M + 15) / 16;
   const bf16_t *x = (const bf16_t*)X, *w = (const bf16_t*)W;
   switch (mb) {
-    case 1: return launch_mb<1>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part, (int*)counters);
-    case 2: return launch_mb<2>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part, (int*)counters);
-    case 3: return launch_mb<3>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part, (int*)counters);
-    default: return launch_mb<4>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part, (int*)counters);
+    case 1: return launch_mb<1>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
+    case 2: return launch_mb<2>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
+    case 3: return launch_mb<3>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
+    default: return launch_mb<4>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
   }
 }

@@ -105,11 +105,152 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(int* __restrict_
   }
 }
 
+// ---- large vocabularies: two stages, so that one row keeps many compute units busy.
+// Stage 1: the row is cut into chunks; each block finds its chunk's maximum (lowest index among
+// equals) and, for sampled rows, the sum of exp((l - chunk max) / tau).
+// Stage 2: one block per row takes the chunk results in chunk order: the global maximum; the total
+// sum (chunk sums rescaled to the global maximum); the chunk the draw falls into; and scans that
+// chunk for the first index whose cumulative weight reaches the draw.
+#define CHUNK_REC 4   // max, index (as float bits), sum, unused
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_stage1_kernel(float* __restrict__ ws, const float* __restrict__ logits,
+                                                                       long row_stride, const float* __restrict__ temperature,
+                                                                       int V, int chunk) {
+  __shared__ float wv[SAMPLE_THREADS / PI_WAVE];
+  __shared__ int wi[SAMPLE_THREADS / PI_WAVE];
+  __shared__ float scratch[16];
+  const int c = blockIdx.x, row = blockIdx.y, tid = threadIdx.x;
+  const float* l = logits + (long)row * row_stride;
+  const int c0 = c * chunk, c1 = min(V, c0 + chunk);
+  ArgMax best = {-INFINITY, 0x7fffffff};
+  for (int i = c0 + tid; i < c1; i += SAMPLE_THREADS) {
+    const float v = l[i];
+    if (v > best.v) best = {v, i};
+  }
+  best = wave_argmax(best);
+  if (tid % PI_WAVE == 0) {
+    wv[tid / PI_WAVE] = best.v;
+    wi[tid / PI_WAVE] = best.i;
+  }
+  __syncthreads();
+  best = {wv[0], wi[0]};
+  for (int w = 1; w < SAMPLE_THREADS / PI_WAVE; ++w) best = better(best, ArgMax{wv[w], wi[w]});
+  const float tau = temperature ? temperature[row] : 0.f;
+  float sum = 0.f;
+  if (tau > 0.f && best.i != 0x7fffffff) {
+    for (int i = c0 + tid; i < c1; i += SAMPLE_THREADS) sum += expf((l[i] - best.v) / tau);
+    sum = block_sum(sum, scratch);
+  }
+  if (tid == 0) {
+    float* rec = ws + ((long)row * gridDim.x + c) * CHUNK_REC;
+    rec[0] = best.v;
+    rec[1] = __int_as_float(best.i);
+    rec[2] = sum;
+  }
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_stage2_kernel(int* __restrict__ out, const float* __restrict__ ws,
+                                                                       const float* __restrict__ logits, long row_stride,
+                                                                       const float* __restrict__ temperature,
+                                                                       const float* __restrict__ uniform, int V, int chunk,
+                                                                       int chunks) {
+  __shared__ float sums[SAMPLE_THREADS];
+  __shared__ int chosen;
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const float* l = logits + (long)row * row_stride;
+  const float* rec = ws + (long)row * chunks * CHUNK_REC;
+  ArgMax best = {-INFINITY, 0x7fffffff};
+  for (int c = 0; c < chunks; ++c) best = better(best, ArgMax{rec[c * CHUNK_REC], __float_as_int(rec[c * CHUNK_REC + 1])});
+  if (best.i == 0x7fffffff) best = {l[0], 0};
+  const float tau = temperature ? temperature[row] : 0.f;
+  if (!(tau > 0.f)) {
+    if (tid == 0) out[row] = best.i;
+    return;
+  }
+  // every thread walks the chunk sums the same way (chunks is small): total, then the chunk of the draw
+  float total = 0.f;
+  for (int c = 0; c < chunks; ++c) {
+    const float m = rec[c * CHUNK_REC];
+    if (m != -INFINITY) total += rec[c * CHUNK_REC + 2] * expf((m - best.v) / tau);
+  }
+  const float target = uniform[row] * total;
+  float before_chunk = 0.f;
+  int pick_chunk = chunks - 1;
+  for (int c = 0; c < chunks; ++c) {
+    const float m = rec[c * CHUNK_REC];
+    const float w = (m != -INFINITY) ? rec[c * CHUNK_REC + 2] * expf((m - best.v) / tau) : 0.f;
+    if (target <= before_chunk + w) {
+      pick_chunk = c;
+      break;
+    }
+    if (c + 1 < chunks) before_chunk += w;
+  }
+  // inside the chunk: each thread owns a contiguous run
+  const int c0 = pick_chunk * chunk, c1 = min(V, c0 + chunk);
+  const int run = (c1 - c0 + SAMPLE_THREADS - 1) / SAMPLE_THREADS;
+  const int r0 = min(c1, c0 + tid * run), r1 = min(c1, r0 + run);
+  float local = 0.f;
+  for (int i = r0; i < r1; ++i) local += expf((l[i] - best.v) / tau);
+  sums[tid] = local;
+  if (tid == 0) chosen = -1;
+  __syncthreads();
+  float before = before_chunk;
+  for (int j = 0; j < tid; ++j) before += sums[j];
+  if ((before < target || (tid == 0 && pick_chunk == 0)) && target <= before + local) {
+    float cum = 0.f;
+    for (int i = r0; i < r1; ++i) {
+      cum += expf((l[i] - best.v) / tau);
+      if (target <= before + cum) {
+        chosen = i;
+        break;
+      }
+    }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    int pick = chosen;
+    if (pick < 0) {
+      // rounding between the chunk sums and the scan: the draw lies at an edge of the chunk.
+      // Below its first weight: the first index with weight; beyond its last: the last one.
+      const bool below = target <= before_chunk;
+      pick = -1;
+      if (below) {
+        for (int i = c0; i < c1 && pick < 0; ++i)
+          if (expf((l[i] - best.v) / tau) > 0.f) pick = i;
+      } else {
+        for (int i = c1 - 1; i >= c0 && pick < 0; --i)
+          if (expf((l[i] - best.v) / tau) > 0.f) pick = i;
+      }
+      if (pick < 0) pick = best.i;
+    }
+    out[row] = pick;
+  }
+}
+
+// Rows of more than `two_stage_from` logits use the two-stage kernels and need `ws`
+// (float32, M * chunks * 4 with chunks = pi_sample_chunks(V)).
+#define TWO_STAGE_FROM 16384
+#define MAX_CHUNKS 64
+
+extern "C" int pi_sample_chunks(int V) {
+  if (V <= TWO_STAGE_FROM) return 0;
+  int chunks = (V + 2047) / 2048;
+  return chunks > MAX_CHUNKS ? MAX_CHUNKS : chunks;
+}
+
 extern "C" int pi_sample(int* out, const float* logits, long row_stride, const float* temperature, const float* uniform,
-                         int M, int V, hipStream_t stream) {
+                         int M, int V, float* ws, long ws_elems, hipStream_t stream) {
   PI_REQUIRE(M >= 0 && V > 0 && row_stride >= V, "sample: bad sizes M=%d V=%d stride=%ld", M, V, row_stride);
   PI_REQUIRE(temperature == nullptr || uniform != nullptr, "sample: temperatures given without uniform numbers");
   if (M == 0) return 0;
-  hipLaunchKernelGGL(sample_kernel, dim3(M), dim3(SAMPLE_THREADS), 0, stream, out, logits, row_stride, temperature, uniform, V);
-  return pi_check_launch("sample");
+  const int chunks = pi_sample_chunks(V);
+  if (chunks == 0 || ws == nullptr || ws_elems < (long)M * chunks * CHUNK_REC || M > 65535) {
+    hipLaunchKernelGGL(sample_kernel, dim3(M), dim3(SAMPLE_THREADS), 0, stream, out, logits, row_stride, temperature, uniform, V);
+    return pi_check_launch("sample");
+  }
+  const int chunk = (V + chunks - 1) / chunks;
+  hipLaunchKernelGGL(sample_stage1_kernel, dim3(chunks, M), dim3(SAMPLE_THREADS), 0, stream, ws, logits, row_stride, temperature, V, chunk);
+  if (pi_check_launch("sample_stage1")) return -1;
+  hipLaunchKernelGGL(sample_stage2_kernel, dim3(M), dim3(SAMPLE_THREADS), 0, stream, out, ws, logits, row_stride, temperature, uniform, V, chunk, chunks);
+  return pi_check_launch("sample_stage2");
 }

@@ -115,8 +115,47 @@ def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float
             raise KernelError(f"rmsnorm: {x.shape[0]} input rows for {M} output rows")
     else:
         _i32(rows, "rmsnorm rows", M)
+    pending = _take_deferred(x)
+    part, splits = (pending.part.data_ptr(), pending.splits) if pending is not None else (None, 0)
     _lib.call("core", "pi_rmsnorm", out.data_ptr(), _dt(out), x.data_ptr(), _ptr(rows), weight.data_ptr(),
-              _dt(weight), float(eps), M, D, _stream())
+              _dt(weight), float(eps), M, D, part, splits, x.shape[0], _stream())
+
+
+# ----------------------------------------------------------------------------- deferred updates
+# A product into the residual stream whose k-range was split over blocks may stay in pieces
+# (a `Partials`) until the next reader of the stream: ``rmsnorm`` folds the sum of the pieces
+# and the residual add into its own pass.  Whoever reads the stream in any other way calls
+# ``materialize`` first.  Only callers that pass ``may_defer=True`` to ``gemm`` ever leave an
+# update pending, and a block arrangement must materialize before it hands the stream to a
+# part that does not read it through ``rmsnorm``.
+def _take_deferred(x: torch.Tensor):
+    from . import fast
+    p = fast.PENDING.pop(x.data_ptr(), None)
+    if p is not None and (p.M, p.N) != tuple(x.shape):
+        fast.reduce_into(x, p, accumulate=True)      # not the tensor it was made for: play safe
+        return None
+    return p
+
+
+def materialize(x: torch.Tensor) -> torch.Tensor:
+    """Apply an update of ``x`` that is still pending, if there is one."""
+    from . import fast
+    p = fast.PENDING.pop(x.data_ptr(), None)
+    if p is not None:
+        fast.reduce_into(x, p, accumulate=True)
+    return x
+
+
+def reset_deferred() -> None:
+    """Forget every pending update (start of a step)."""
+    from . import fast
+    fast.PENDING.clear()
+
+
+def discard_deferred(x: torch.Tensor) -> None:
+    """Forget a pending update of ``x`` (the stream is not read again)."""
+    from . import fast
+    fast.PENDING.pop(x.data_ptr(), None)
 
 
 def swiglu(out: torch.Tensor, gate_up: torch.Tensor, block: int = 0) -> None:
@@ -150,8 +189,12 @@ def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate_up: torch.Tensor, blo
     swiglu(out, gu, block)
 
 
-def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, accumulate: bool = False) -> None:
-    """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation."""
+def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, accumulate: bool = False,
+         may_defer: bool = False) -> None:
+    """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation.
+
+    ``may_defer`` (with ``accumulate``): the caller promises that ``out`` is next read by
+    ``rmsnorm`` or ``materialize``; a product that was split over k may then stay in pieces."""
     _gpu(out, a, w)
     if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
         raise KernelError("gemm: operands must be 2-D")
@@ -164,9 +207,11 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, accumulate: bool =
     lda, ldw, ldc = _rows(a, "gemm a"), _rows(w, "gemm w"), _rows(out, "gemm out")
     if M == 0:
         return
+    if accumulate:
+        materialize(out)
     if _FAST and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
         from . import fast
-        if fast.gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc):
+        if fast.gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc, may_defer and accumulate and out.is_contiguous()):
             return
     _lib.call("core", "pi_gemm_general", out.data_ptr(), _dt(out), ldc, a.data_ptr(), _dt(a), lda, w.data_ptr(),
               _dt(w), ldw, M, N, K, int(accumulate), _stream())
@@ -183,14 +228,31 @@ def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, hd: int
     return k_cache.shape[0]
 
 
+def qkv_projection(h: torch.Tensor, w_qkv: torch.Tensor, dtype: torch.dtype):
+    """h @ w_qkv^T for the attention mixer: a tensor [T, N] in ``dtype``, or - when the
+    product was split over k - its pieces (``fast.Partials``), which ``rope_kv_write`` sums
+    on the fly so that the rotation sees float32 values."""
+    if _FAST and h.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and h.is_cuda:
+        from . import fast
+        p = fast.gemm_pieces(h, w_qkv)
+        if p is not None:
+            return p
+    out = torch.empty((h.shape[0], w_qkv.shape[0]), dtype=dtype, device=h.device)
+    gemm(out, h, w_qkv)
+    return out
+
+
 def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.Tensor], positions: torch.Tensor,
                   req_of_token: torch.Tensor, rotary, num_heads: int, num_kv_heads: int, head_dim: int,
                   k_cache: Optional[torch.Tensor], v_cache: Optional[torch.Tensor],
-                  block_table: Optional[torch.Tensor], page_size: int) -> None:
+                  block_table: Optional[torch.Tensor], page_size: int, pieces=None, write_kv: Optional[bool] = None) -> None:
     """Rotate q in place by each token's position; rotate k and store k, v into the pages.
 
     ``rotary`` = (inv_freq float32 [R/2], R, interleaved) or None for no rotation.
     ``k``/``v`` None: queries only (the layer reads a cache that another one writes).
+    ``pieces``: the q|k|v projection still split over k (``fast.Partials`` with columns
+    [q heads | k heads | v heads]); then ``q`` is the output buffer for the rotated queries and
+    ``k``/``v`` are not given (``write_kv`` says whether the cache is written).
     """
     _gpu(q, k, v, positions, req_of_token, k_cache, v_cache, block_table)
     T = q.shape[0]
@@ -198,6 +260,20 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
     if q.shape[1] != num_heads * head_dim:
         raise KernelError(f"rope: q has {q.shape[1]} columns, expected {num_heads * head_dim}")
     _i32(positions, "positions", T)
+    if pieces is not None:
+        write = bool(write_kv)
+        inv_freq, rdim, inter = (None, 0, False) if rotary is None else rotary
+        q_size, kv_size = num_heads * head_dim, num_kv_heads * head_dim
+        if pieces.M != T or pieces.N < q_size + (2 * kv_size if write else 0):
+            raise KernelError(f"rope: pieces [{pieces.M}, {pieces.N}] do not hold q, k, v of {T} tokens")
+        pages = _check_cache(k_cache, v_cache, num_kv_heads, head_dim, page_size, q.dtype) if write else 0
+        _lib.call(
+            "core", "pi_rope_kv_write", q.data_ptr(), _rows(q, "q"), None, 0, None, 0, _dt(q), positions.data_ptr(),
+            _ptr(req_of_token) if write else None, _ptr(inv_freq), rdim, int(bool(inter)), T, num_heads, num_kv_heads,
+            head_dim, int(write), _ptr(k_cache) if write else None, _ptr(v_cache) if write else None,
+            _ptr(block_table) if write else None, block_table.shape[1] if write else 0, page_size if write else 0, pages,
+            pieces.part.data_ptr(), pieces.splits, pieces.N, 0, q_size, q_size + kv_size, _stream())
+        return
     write = k is not None
     inv_freq, rdim, inter = (None, 0, False) if rotary is None else rotary
     if inv_freq is not None and (inv_freq.dtype != torch.float32 or inv_freq.numel() != rdim // 2 or not inv_freq.is_contiguous()):
@@ -217,7 +293,7 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
         _rows(v, "v") if write else 0, _dt(q), positions.data_ptr(), _ptr(req_of_token) if write else None,
         _ptr(inv_freq), rdim, int(bool(inter)), T, num_heads, num_kv_heads, head_dim, int(write),
         _ptr(k_cache) if write else None, _ptr(v_cache) if write else None, _ptr(block_table) if write else None,
-        block_table.shape[1] if write else 0, page_size if write else 0, pages, _stream())
+        block_table.shape[1] if write else 0, page_size if write else 0, pages, None, 0, 0, 0, 0, 0, _stream())
 
 
 def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -266,8 +342,14 @@ def sample(out: torch.Tensor, logits: torch.Tensor, temperature: Optional[torch.
             raise KernelError(f"sample: {what} must be contiguous float32 [{M}]")
     if temperature is not None and uniform is None:
         raise KernelError("sample: temperatures given without uniform numbers")
+    ws = _SAMPLE_WS.get(logits.device)
+    if ws is None:
+        ws = _SAMPLE_WS[logits.device] = torch.empty(1 << 18, dtype=torch.float32, device=logits.device)
     _lib.call("core", "pi_sample", out.data_ptr(), logits.data_ptr(), _rows(logits, "logits"), _ptr(temperature),
-              _ptr(uniform), M, V, _stream())
+              _ptr(uniform), M, V, ws.data_ptr(), ws.numel(), _stream())
+
+
+_SAMPLE_WS: dict = {}
 
 
 # ----------------------------------------------------------------------------- work lists

@@ -14,19 +14,20 @@ P, I, L, F = c_void_p, c_int, c_long, c_float
 _SIGNATURES = {
     "core": {
         "pi_embedding": [P, P, I, P, I, I, I, P],
-        "pi_rmsnorm": [P, I, P, P, P, I, F, I, I, P],
+        "pi_rmsnorm": [P, I, P, P, P, I, F, I, I, P, I, L, P],
         "pi_swiglu": [P, P, I, I, I, I, P],
-        "pi_rope_kv_write": [P, L, P, L, P, L, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, I, L, P],
+        "pi_rope_kv_write": [P, L, P, L, P, L, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, I, I, I, I, P],
         "pi_gemm_general": [P, I, L, P, I, L, P, I, L, I, I, I, I, P],
         "pi_paged_attention_general": [P, L, P, L, P, P, I, P, I, P, P, I, I, I, I, I, F, I, L, P],
-        "pi_sample": [P, P, L, P, P, I, I, P],
+        "pi_sample": [P, P, L, P, P, I, I, P, L, P],
     },
     "bf16": {
         "pi_gemm_mfma": [P, I, L, P, L, P, L, I, I, I, P],
-        "pi_gemm_skinny": [P, I, L, P, L, P, L, I, I, I, I, P, L, P, L, P],
+        "pi_gemm_skinny": [P, I, L, P, L, P, L, I, I, I, I, P, L, P, P],
+        "pi_splitk_reduce": [P, I, L, P, I, I, I, P],
         "pi_attention_tile_rows": [I, I, I],
         "pi_attention_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, P, I, I, I, I, I, F, I, L, P],
-        "pi_attention_decode": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, P, L, P],
+        "pi_attention_decode": [P, L, P, L, P, P, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, P],
     },
 }
 

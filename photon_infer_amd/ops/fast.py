@@ -13,6 +13,8 @@ Which kernel takes what:
 """
 from __future__ import annotations
 
+import ctypes
+from dataclasses import dataclass
 from typing import Dict, Optional
 
 import numpy as np
@@ -25,21 +27,34 @@ SKINNY_MAX_ROWS = 64
 ROWS_PER_BLOCK = 32            # weight rows per block of the skinny kernel
 TARGET_BLOCKS = 512            # blocks wanted in flight to keep HBM busy
 GEMM_PART_FLOATS = 4 << 20     # k-split partial sums of the skinny kernel
-GEMM_COUNTERS = 8192
 ATTN_PART_FLOATS = 4 << 20     # key-split partial results of decode attention
-ATTN_COUNTERS = 1 << 16
 MAX_DECODE_SPLITS = 64
 
 
 class _Workspace:
-    """Scratch the kernels share on one device: partial sums and self-resetting counters.
-    Kernels on one stream run one after another, so one set is enough."""
+    """Scratch the kernels share on one device: the pieces of products split over k and of
+    attention split over keys.  Kernels on one stream run one after another, so one set is
+    enough; a product left in pieces (see ``Partials``) owns the product scratch until it is
+    consumed."""
 
     def __init__(self, device):
         self.gemm_part = torch.empty(GEMM_PART_FLOATS, dtype=torch.float32, device=device)
-        self.gemm_counters = torch.zeros(GEMM_COUNTERS, dtype=torch.int32, device=device)
         self.attn_part = torch.empty(ATTN_PART_FLOATS, dtype=torch.float32, device=device)
-        self.attn_counters = torch.zeros(ATTN_COUNTERS, dtype=torch.int32, device=device)
+        self.splits_out = ctypes.c_int(0)
+
+
+@dataclass
+class Partials:
+    """A product [M, N] whose k-range was split: ``part`` holds float32 [splits, M, N]."""
+
+    part: torch.Tensor
+    splits: int
+    M: int
+    N: int
+
+
+# updates of a residual stream that are still in pieces, keyed by the stream's address
+PENDING: Dict[int, Partials] = {}
 
 
 _WORKSPACES: Dict[torch.device, _Workspace] = {}
@@ -65,22 +80,34 @@ def _skinny_splits(M: int, N: int, K: int) -> int:
     splits = max(1, min(-(-TARGET_BLOCKS // groups), K // 256))
     while splits > 1 and splits * M * N > GEMM_PART_FLOATS:
         splits -= 1
-    return splits if groups <= GEMM_COUNTERS else 1
+    return splits
 
 
-def _run_gemm(out, epilogue: int, ldc: int, a, w, M: int, N: int, K: int, lda: int, ldw: int) -> None:
-    if M <= SKINNY_MAX_ROWS:
-        splits = 1 if epilogue == EPI_SWIGLU else _skinny_splits(M, N, K)
-        ws = workspace(a.device)
-        _lib.call("bf16", "pi_gemm_skinny", out.data_ptr(), epilogue, ldc, a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K,
-                  splits, ws.gemm_part.data_ptr(), ws.gemm_part.numel(), ws.gemm_counters.data_ptr(),
-                  ws.gemm_counters.numel(), _stream())
-    else:
-        _lib.call("bf16", "pi_gemm_mfma", out.data_ptr(), epilogue, ldc, a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K,
-                  _stream())
+def _flush_pending() -> None:
+    """The product scratch is about to be reused: finish whatever still lives in it."""
+    for ptr in list(PENDING):
+        p = PENDING.pop(ptr)
+        _lib.call("bf16", "pi_splitk_reduce", ptr, EPI_ACCUM, p.N, p.part.data_ptr(), p.splits, p.M, p.N, _stream())
 
 
-def gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc) -> bool:
+def _skinny(out_ptr: int, epilogue: int, ldc: int, a, w, M, N, K, lda, ldw, splits: int) -> Optional[Partials]:
+    """Run the weight-streaming kernel; returns the pieces when the product was split."""
+    ws = workspace(a.device)
+    if splits > 1:
+        _flush_pending()
+    _lib.call("bf16", "pi_gemm_skinny", out_ptr, epilogue, ldc, a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K, splits,
+              ws.gemm_part.data_ptr(), ws.gemm_part.numel(), ctypes.byref(ws.splits_out), _stream())
+    made = ws.splits_out.value
+    return Partials(ws.gemm_part, made, M, N) if made > 1 else None
+
+
+def reduce_into(out: torch.Tensor, p: Partials, accumulate: bool) -> None:
+    epilogue = EPI_ACCUM if accumulate else (EPI_BF16 if out.dtype == torch.bfloat16 else EPI_F32)
+    _lib.call("bf16", "pi_splitk_reduce", out.data_ptr(), epilogue, out.stride(0), p.part.data_ptr(), p.splits, p.M, p.N,
+              _stream())
+
+
+def gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc, may_defer=False) -> bool:
     if not _gemm_ok(a, w, K, lda, ldw):
         return False
     if accumulate:
@@ -91,15 +118,42 @@ def gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc) -> bool:
         epilogue = EPI_F32
     else:
         return False
-    _run_gemm(out, epilogue, ldc, a, w, M, N, K, lda, ldw)
+    if M > SKINNY_MAX_ROWS:
+        _lib.call("bf16", "pi_gemm_mfma", out.data_ptr(), epilogue, ldc, a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K,
+                  _stream())
+        return True
+    pieces = _skinny(out.data_ptr(), epilogue, ldc, a, w, M, N, K, lda, ldw, _skinny_splits(M, N, K))
+    if pieces is not None:
+        if may_defer:
+            PENDING[out.data_ptr()] = pieces          # the next norm of this stream adds them
+        else:
+            _lib.call("bf16", "pi_splitk_reduce", out.data_ptr(), epilogue, ldc, pieces.part.data_ptr(), pieces.splits,
+                      M, N, _stream())
     return True
+
+
+def gemm_pieces(a, w) -> Optional[Partials]:
+    """a @ w^T left in pieces, if this product is one the weight-streaming kernel would split."""
+    M, K = a.shape
+    N = w.shape[0]
+    lda, ldw = a.stride(0) if M > 1 else K, w.stride(0)
+    if M > SKINNY_MAX_ROWS or not _gemm_ok(a, w, K, lda, ldw) or a.stride(1) != 1 or w.stride(1) != 1:
+        return None
+    splits = _skinny_splits(M, N, K)
+    if splits <= 1:
+        return None
+    return _skinny(0, EPI_F32, N, a, w, M, N, K, lda, ldw, splits)
 
 
 def gemm_swiglu(out, a, w, M, N, K, lda, ldw) -> bool:
     """``w`` [N = 2I, K] with gate / up rows interleaved in blocks of 16; out [M, I] bfloat16."""
     if not _gemm_ok(a, w, K, lda, ldw) or N % 32 or out.dtype != torch.bfloat16:
         return False
-    _run_gemm(out, EPI_SWIGLU, out.stride(0), a, w, M, N, K, lda, ldw)
+    if M > SKINNY_MAX_ROWS:
+        _lib.call("bf16", "pi_gemm_mfma", out.data_ptr(), EPI_SWIGLU, out.stride(0), a.data_ptr(), lda, w.data_ptr(), ldw,
+                  M, N, K, _stream())
+    else:
+        _skinny(out.data_ptr(), EPI_SWIGLU, out.stride(0), a, w, M, N, K, lda, ldw, 1)
     return True
 
 
@@ -151,13 +205,11 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
         ws = workspace(q.device)
         while splits > 1 and R * num_heads * splits * (head_dim + 4) > ws.attn_part.numel():
             splits -= 1
-        if R * num_kv_heads <= ws.attn_counters.numel():
-            _lib.call("bf16", "pi_attention_decode", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
-                      k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
-                      ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), R, num_heads, num_kv_heads, head_dim, page_size,
-                      float(scale), int(window), pages, splits, ws.attn_part.data_ptr(), ws.attn_part.numel(),
-                      ws.attn_counters.data_ptr(), ws.attn_counters.numel(), _stream())
-            return True
+        _lib.call("bf16", "pi_attention_decode", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
+                  k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
+                  ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), R, num_heads, num_kv_heads, head_dim, page_size,
+                  float(scale), int(window), pages, splits, ws.attn_part.data_ptr(), ws.attn_part.numel(), _stream())
+        return True
     tile_rows = attention_tile_rows(num_heads, num_kv_heads, head_dim)
     if tile_rows < 1:
         return False

@@ -77,29 +77,38 @@ class PagedAttention(Mixer):
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
         T = h.shape[0]
-        qkv = torch.empty((T, self.w_qkv.shape[0]), dtype=self.dtype, device=h.device)
-        ops.gemm(qkv, h, self.w_qkv)
-        q = qkv[:, : self.q_size]
         writes = self.own_kv and cache.writes
-        k = qkv[:, self.q_size : self.q_size + self.kv_size] if self.own_kv else None
-        v = qkv[:, self.q_size + self.kv_size :] if self.own_kv else None
         rotary = self.position.rotary_params() if self.position is not None else None
-        if self.position is not None and rotary is None:
-            self.position.apply(q, k, ctx)
+        fused_position = self.position is None or rotary is not None
         table = ctx.block_tables[cache.group]
-        ops.rope_kv_write(
-            q, k if writes else None, v if writes else None,
-            ctx.positions, ctx.req_of_token,
-            rotary, self.num_heads, self.num_kv_heads, self.head_dim,
-            cache.k, cache.v, table, cache.page_size,
-        )
+        qkv = ops.qkv_projection(h, self.w_qkv, self.dtype) if fused_position else None
+        if qkv is not None and not isinstance(qkv, torch.Tensor):
+            # the projection is still in pieces (split over k): the rotation kernel sums them
+            q = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
+            ops.rope_kv_write(q, None, None, ctx.positions, ctx.req_of_token, rotary, self.num_heads,
+                              self.num_kv_heads, self.head_dim, cache.k, cache.v, table, cache.page_size,
+                              pieces=qkv, write_kv=writes)
+        else:
+            if qkv is None:
+                qkv = torch.empty((T, self.w_qkv.shape[0]), dtype=self.dtype, device=h.device)
+                ops.gemm(qkv, h, self.w_qkv)
+            q = qkv[:, : self.q_size]
+            k = qkv[:, self.q_size : self.q_size + self.kv_size] if self.own_kv else None
+            v = qkv[:, self.q_size + self.kv_size :] if self.own_kv else None
+            if not fused_position:
+                self.position.apply(q, k, ctx)
+            ops.rope_kv_write(
+                q, k if writes else None, v if writes else None, ctx.positions, ctx.req_of_token,
+                rotary, self.num_heads, self.num_kv_heads, self.head_dim, cache.k, cache.v, table, cache.page_size,
+            )
         attn = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
         ops.paged_attention(
             attn, q, cache.k, cache.v, table, ctx,
             self.num_heads, self.num_kv_heads, self.head_dim, cache.page_size,
             self.scale, self.window or 0,
         )
-        ops.gemm(x, attn, self.w_o, accumulate=True)
+        # the block's next norm reads x, so the product may stay in pieces until then
+        ops.gemm(x, attn, self.w_o, accumulate=True, may_defer=True)
 
 
 MIXERS.register("attention", PagedAttention)

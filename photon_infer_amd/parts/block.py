@@ -10,6 +10,7 @@ from typing import Dict, List, Tuple
 
 import torch
 
+from .. import ops
 from ..weights.loader import TensorSpec
 from .base import BLOCKS, Block, FeedForward, LayerCache, Mixer, Norm, Part, StepContext
 
@@ -31,7 +32,14 @@ class PreNormBlock(Block):
             part.load({n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}, dtype, device)
 
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
+        # A mixer or feed-forward may leave its update of x in pieces for the next norm to add
+        # (ops.gemm(..., may_defer=True)).  A norm that does not go through ops.rmsnorm gets
+        # the finished stream; mixers and feed-forwards always do, since a norm runs before them.
+        if not getattr(self.norm1, "consumes_deferred", False):
+            ops.materialize(x)
         self.mixer.forward(self.norm1.forward(x), x, ctx, cache)
+        if not getattr(self.norm2, "consumes_deferred", False):
+            ops.materialize(x)
         self.ffn.forward(self.norm2.forward(x), x, ctx)
 
 

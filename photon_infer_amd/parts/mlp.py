@@ -55,7 +55,7 @@ class SwiGLU(FeedForward):
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
         act = torch.empty((h.shape[0], self.intermediate_size), dtype=self.dtype, device=h.device)
         ops.gemm_swiglu(act, h, self.w_gate_up, self.interleave)
-        ops.gemm(x, act, self.w_down, accumulate=True)
+        ops.gemm(x, act, self.w_down, accumulate=True, may_defer=True)   # the next norm reads x
 
 
 FEED_FORWARDS.register("swiglu", SwiGLU)

@@ -13,6 +13,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 
 import torch
 
+from .. import ops
 from ..errors import ConfigError
 from ..weights.loader import TensorSpec
 from .base import Block, KVCacheSpec, LayerCache, Norm, StateSpec, StepContext
@@ -134,9 +135,13 @@ class DecoderModel:
     def forward(self, ctx: StepContext, caches: Sequence[LayerCache]) -> Optional[torch.Tensor]:
         """Run the step's tokens through the run order; float32 logits [M, vocab] at
         ``ctx.logit_rows`` (None when no row is wanted)."""
+        ops.reset_deferred()               # nothing of an earlier (failed) step may linger
         x = self.embedding.forward(ctx.token_ids)
         for i, entry in enumerate(self.spec.run_order):
             self.blocks[entry.layer].forward(x, ctx, caches[i])
         if ctx.logit_rows.shape[0] == 0:
+            ops.discard_deferred(x)        # the stream is not read again
             return None
+        if not getattr(self.final_norm, "consumes_deferred", False):
+            ops.materialize(x)
         return self.head.forward(self.final_norm.forward(x, rows=ctx.logit_rows))

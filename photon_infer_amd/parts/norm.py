@@ -17,6 +17,8 @@ from .base import NORMS, Norm
 
 
 class RMSNorm(Norm):
+    consumes_deferred = True   # reads the stream through ops.rmsnorm, which adds a pending update
+
     def __init__(self, dim: int, eps: float):
         self.dim = int(dim)
         self.eps = float(eps)

@@ -66,6 +66,8 @@ def test_swiglu_part(dtype):
     x0 = torch.randn(T, D, generator=gen(6))
     x = x0.clone().to(DEV)
     ffn.forward(h.to(DEV), x, None)
+    from photon_infer_amd import ops
+    ops.materialize(x)          # the product may still be in pieces for a norm to add
     Wr = {k: v.to(dtype).float() for k, v in W.items()}
     rd = (lambda t: t) if dtype == F32 else P.bf16_round
     act = rd(P.swiglu(rd(P.linear(h.float(), Wr["gate_proj.weight"])), rd(P.linear(h.float(), Wr["up_proj.weight"]))))
@@ -78,6 +80,7 @@ def test_swiglu_part(dtype):
 def test_attention_part(dtype, window):
     """The mixer alone: projections, rotation, cache write, attention over pages, output
     projection into the residual - in two steps, so the second reads what the first wrote."""
+    from photon_infer_amd import ops
     from photon_infer_amd.parts import MIXERS, POSITION_ENCODINGS, KVCacheSpec, LayerCache
     D, nh, nkv, hd, page = 80, 6, 2, 32, 4
     rope = POSITION_ENCODINGS.make("rope", head_dim=hd, theta=10000.0)
@@ -95,7 +98,9 @@ def test_attention_part(dtype, window):
     for lo, hi in ((0, first), (first, S)):
         ctx = attention_ctx([hi - lo], [hi], dtype)
         ctx.block_tables = {0: table}
-        attn.forward(h[lo:hi].to(DEV), x[lo:hi], ctx, cache)
+        xs = x[lo:hi]
+        attn.forward(h[lo:hi].to(DEV), xs, ctx, cache)
+        ops.materialize(xs)
     Wr = {k: v.to(dtype).float() for k, v in W.items()}
     rd = (lambda t: t) if dtype == F32 else P.bf16_round
     f = P.rope_frequencies(hd, 10000.0, None)
