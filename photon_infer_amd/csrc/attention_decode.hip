@@ -80,19 +80,32 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(bf16_t* __restric
   const int head = blockIdx.x, r = blockIdx.y;
   const int rec = HD + 4;
   const float* base = part + ((long)r * nh + head) * splits * rec;
-  float m_tot = -INFINITY;
-  for (int s = 0; s < splits; ++s) m_tot = fmaxf(m_tot, base[s * rec + HD]);
+  // lane s holds range s (splits <= 64): maxima, weights and the total in parallel
+  const float ms = lane < splits ? base[lane * rec + HD] : -INFINITY;
+  const float ls = lane < splits ? base[lane * rec + HD + 1] : 0.f;
+  const float m_tot = wave_max(ms);
+  const float w = (ms == -INFINITY) ? 0.f : expf(ms - m_tot);
   float l_tot = 0.f;
   float acc[HD / 64];
 #pragma unroll
   for (int i = 0; i < HD / 64; ++i) acc[i] = 0.f;
-  for (int s = 0; s < splits; ++s) {
-    const float ms = base[s * rec + HD];
-    if (ms == -INFINITY) continue;
-    const float w = expf(ms - m_tot);
-    l_tot += w * base[s * rec + HD + 1];
+  // ranges in order; eight loads in flight at a time
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float o[8][HD / 64], ws[8];
 #pragma unroll
-    for (int i = 0; i < HD / 64; ++i) acc[i] += w * base[s * rec + lane + i * 64];
+    for (int u = 0; u < 8; ++u) {
+      const int s = s0 + u;
+      ws[u] = __shfl(w, s < splits ? s : 0, 64);
+      if (s >= splits) ws[u] = 0.f;
+#pragma unroll
+      for (int i = 0; i < HD / 64; ++i) o[u][i] = (s < splits) ? base[s * rec + lane + i * 64] : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      l_tot += ws[u] * __shfl(ls, (s0 + u < splits) ? s0 + u : 0, 64);
+#pragma unroll
+      for (int i = 0; i < HD / 64; ++i) acc[i] += ws[u] * o[u][i];
+    }
   }
   const float inv = 1.0f / l_tot;
   bf16_t* o = out + (long)q_start[r] * out_stride + (long)head * HD;
@@ -108,7 +121,7 @@ extern "C" int pi_attention_decode(void* out, long out_stride, const void* q, lo
   PI_REQUIRE(R > 0 && nh > 0 && nkv > 0 && nh % nkv == 0 && nh / nkv <= 16, "attention_decode: needs 1..16 heads per kv head, got %d / %d", nh, nkv);
   PI_REQUIRE(hd == 64 || hd == 128, "attention_decode: head_dim %d is not 64 or 128", hd);
   PI_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_decode: page size %d must be a multiple of 16", page_size);
-  PI_REQUIRE(splits >= 1 && splits <= 1024 && R <= 65535 && nkv <= 65535, "attention_decode: bad grid (%d ranges, %d requests, %d kv heads)", splits, R, nkv);
+  PI_REQUIRE(splits >= 1 && splits <= 64 && R <= 65535 && nkv <= 65535, "attention_decode: bad grid (%d ranges, %d requests, %d kv heads)", splits, R, nkv);
   PI_REQUIRE(out_stride % 4 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "attention_decode: q / out rows must be 16- / 8-byte aligned");
   if (splits > 1)
     PI_REQUIRE(part && part_elems >= (long)R * nh * splits * (hd + 4), "attention_decode: workspace too small for %d ranges", splits);

@@ -54,7 +54,14 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ x, cons
     const float* pr = part + r * D;
     for (int i = threadIdx.x; i < D; i += blockDim.x) {
       float v = xr[i];
-      for (int s = 0; s < splits; ++s) v += pr[s * part_stride + i];
+      // eight pieces at a time: the loads go out together, the adds keep the split order
+      for (int s0 = 0; s0 < splits; s0 += 8) {
+        float t[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) t[u] = (s0 + u < splits) ? pr[(s0 + u) * part_stride + i] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v += t[u];
+      }
       xr[i] = v;               // the same thread reads it back below
       ss += v * v;
     }
@@ -76,7 +83,8 @@ extern "C" int pi_rmsnorm(void* out, int out_dtype, float* x, const int* rows, c
   PI_REQUIRE(M >= 0 && D > 0, "rmsnorm: bad sizes M=%d D=%d", M, D);
   PI_REQUIRE(part == nullptr || (splits >= 1 && x_rows > 0), "rmsnorm: bad split description (%d splits, %ld rows)", splits, x_rows);
   if (M == 0) return 0;
-  const int threads = D >= 1024 ? 256 : (D >= 256 ? 128 : 64);
+  // few rows: many threads per row, so that a row's loads are all in flight at once
+  const int threads = (D >= 2048 && M <= 256) ? 1024 : (D >= 1024 ? 256 : (D >= 256 ? 128 : 64));
   const long stride = x_rows * (long)D;
 #define LAUNCH(TO, TW) \
   hipLaunchKernelGGL((rmsnorm_kernel<TO, TW>), dim3(M), dim3(threads), 0, stream, (TO*)out, x, rows, (const TW*)w, eps, D, part, splits, stride)

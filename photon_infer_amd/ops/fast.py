@@ -28,7 +28,7 @@ ROWS_PER_BLOCK = 32            # weight rows per block of the skinny kernel
 TARGET_BLOCKS = 512            # blocks wanted in flight to keep HBM busy
 GEMM_PART_FLOATS = 4 << 20     # k-split partial sums of the skinny kernel
 ATTN_PART_FLOATS = 4 << 20     # key-split partial results of decode attention
-MAX_DECODE_SPLITS = 64
+MAX_DECODE_SPLITS = 32
 
 
 class _Workspace:
@@ -187,9 +187,9 @@ def _tiles(ctx, tile_rows: int, device):
 def decode_splits(R: int, num_kv_heads: int, max_kv_len: Optional[int] = None) -> int:
     """Key ranges per (request, kv head): enough waves to fill the chip, no more than the
     keys are worth."""
-    splits = max(1, min(MAX_DECODE_SPLITS, -(-1024 // (R * num_kv_heads))))
+    splits = max(1, min(MAX_DECODE_SPLITS, -(-2048 // (R * num_kv_heads))))
     if max_kv_len is not None:
-        splits = min(splits, max(1, -(-max_kv_len // 64)))
+        splits = min(splits, max(1, -(-max_kv_len // 128)))
     return splits
 
 
