@@ -27,8 +27,8 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
 
   AttnState<HD, 1> st;
   attn_init(st);
-  const bool valid = lr < G;
-  st.pos[0] = valid ? p : -1;
+  const bool valid = lr < G;     // the other columns are padding: computed on zeros, never stored
+  st.pos[0] = p;
   st.lo[0] = lo;
   attn_load_q(st, 0, q, q_stride, row, g * G + lr, valid, lane);
 
@@ -38,8 +38,8 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   const int per = (chunks + splits - 1) / splits;
   const int c0 = first_chunk + split * per;
   const int c1 = min(last_chunk + 1, c0 + per);
-  for (int c = c0; c < c1; ++c)
-    attn_chunk<HD, 1>(st, c * 32, k_cache, v_cache, bt, table_width, kv_len, nkv, g, page_size, num_pages, scale, lane);
+  attn_walk<HD, 1>(st, c0, c1, (lo + 31) / 32, (p + 1) / 32 - 1, k_cache, v_cache, bt, table_width, kv_len, nkv, g,
+                   page_size, num_pages, scale * PI_LOG2E, lane);
 
   const int head = g * G + lr;
   if (splits == 1) {
@@ -84,7 +84,7 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(bf16_t* __restric
   const float ms = lane < splits ? base[lane * rec + HD] : -INFINITY;
   const float ls = lane < splits ? base[lane * rec + HD + 1] : 0.f;
   const float m_tot = wave_max(ms);
-  const float w = (ms == -INFINITY) ? 0.f : expf(ms - m_tot);
+  const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - m_tot);   // maxima are in the base-2 scale
   float l_tot = 0.f;
   float acc[HD / 64];
 #pragma unroll

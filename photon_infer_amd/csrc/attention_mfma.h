@@ -13,18 +13,32 @@
 // 8-byte loads.  Running maximum, running sum and the rescaling factor belong to a column,
 // i.e. to lane % 16, replicated over the four lane groups.
 //
-// Scores, softmax and both accumulations are float32; P is rounded to bfloat16 for the
-// second product, the sum of P is taken before rounding.
+// Scores, softmax and both accumulations are float32.  The exponential is taken in base 2
+// (scores are scaled by scale * log2(e) once, then v_exp_f32), so the running maximum is kept
+// in that scale too.  P is rounded to bfloat16 for the second product; the sum of P is taken
+// before rounding.
+//
+// The keys and values of a chunk are loaded into registers by attn_load and consumed by
+// attn_compute, so a caller can have the next chunk's loads in flight while it computes.
 #pragma once
 #include "mfma.h"
+
+#define PI_LOG2E 1.4426950408889634f
 
 template <int HD, int CB>
 struct AttnState {
   Frag q[CB][HD / 32];
   f32x4_t o[HD / 16][CB];
-  float m[CB], l[CB];
-  int pos[CB];   // last visible key of the column; -1: the column is padding
-  int lo[CB];    // first visible key of the column
+  float m[CB], l[CB];   // running maximum (base-2 scale) and running sum per column
+  int pos[CB];          // last visible key of the column
+  int lo[CB];           // first visible key of the column
+};
+
+template <int HD>
+struct KVChunk {
+  Frag k[2][HD / 32];   // key tiles: rows key0 + lane % 16
+  Frag v[HD / 16];      // value rows d = db*16 + lane % 16; keys (lane/16)*4..+3 of both tiles
+  bool have[2];
 };
 
 template <int HD, int CB>
@@ -38,59 +52,50 @@ __device__ inline void attn_init(AttnState<HD, CB>& st) {
   }
 }
 
-// One chunk of 32 keys starting at k0 (a multiple of 32).  `bt` is the request's block-table
-// row, `kv_len` the number of keys its pages hold.  page_size is a multiple of 16.
-template <int HD, int CB>
-__device__ inline void attn_chunk(AttnState<HD, CB>& st, int k0, const bf16_t* __restrict__ k_cache,
-                                  const bf16_t* __restrict__ v_cache, const int* __restrict__ bt, int table_width,
-                                  int kv_len, int nkv, int g, int page_size, long num_pages, float scale, int lane) {
+// Issue the loads of the 32 keys starting at k0 (a multiple of 32).  `bt` is the request's
+// block-table row, `kv_len` the number of keys its pages hold; page_size is a multiple of 16.
+// A tile whose page is missing (beyond the length, or given back by a window) loads zeros.
+template <int HD>
+__device__ inline void attn_load(KVChunk<HD>& kv, int k0, const bf16_t* __restrict__ k_cache,
+                                 const bf16_t* __restrict__ v_cache, const int* __restrict__ bt, int table_width,
+                                 int kv_len, int nkv, int g, int page_size, long num_pages, int lane) {
   const int lr = lane % 16, lg = lane / 16;
-  long kbase[2], vbase[2];
-  bool have[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const int key0 = k0 + t * 16;
     const int blk = key0 / page_size;
     long page = -1;
     if (key0 < kv_len && blk < table_width) page = bt[blk];
-    have[t] = page >= 0 && page < num_pages;
-    const long pg = have[t] ? page : 0;
+    kv.have[t] = page >= 0 && page < num_pages;
+    const long pg = kv.have[t] ? page : 0;
     const int slot = key0 % page_size;
-    kbase[t] = ((pg * nkv + g) * page_size + slot) * HD;
-    vbase[t] = (pg * nkv + g) * (long)page_size * HD + slot;
+    const bf16_t* kp = k_cache + ((pg * nkv + g) * page_size + slot + lr) * HD + lg * 8;
+    const bf16_t* vp = v_cache + (pg * nkv + g) * (long)page_size * HD + slot + (long)lr * page_size + lg * 4;
+#pragma unroll
+    for (int ks = 0; ks < HD / 32; ++ks) kv.k[t][ks] = kv.have[t] ? load_frag(kp + ks * 32) : zero_frag();
+#pragma unroll
+    for (int db = 0; db < HD / 16; ++db)
+      kv.v[db].d[t] = kv.have[t] ? *reinterpret_cast<const uint2*>(vp + (long)db * 16 * page_size) : make_uint2(0u, 0u);
   }
+}
 
-  // S^T = K . Q^T
+// Fold one loaded chunk into the state.  `masked`: some key of the chunk may be invisible to
+// some column (causal edge, window edge, missing tile); otherwise the per-key tests are skipped.
+template <int HD, int CB>
+__device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv, int k0, float scale_log2, bool masked,
+                                    int lane) {
+  const int lg = lane / 16;
   f32x4_t s[2][CB];
 #pragma unroll
-  for (int t = 0; t < 2; ++t) {
-    Frag a[HD / 32];
-#pragma unroll
-    for (int ks = 0; ks < HD / 32; ++ks)
-      a[ks] = have[t] ? load_frag(k_cache + kbase[t] + (long)lr * HD + ks * 32 + lg * 8) : zero_frag();
+  for (int t = 0; t < 2; ++t)
 #pragma unroll
     for (int c = 0; c < CB; ++c) {
       f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < HD / 32; ++ks) acc = mfma16(a[ks], st.q[c][ks], acc);
+      for (int ks = 0; ks < HD / 32; ++ks) acc = mfma16(kv.k[t][ks], st.q[c][ks], acc);
       s[t][c] = acc;
     }
-  }
 
-  // V^T fragments: rows d = db*16 + lr, keys lg*4..lg*4+3 of each tile
-  Frag va[HD / 16];
-#pragma unroll
-  for (int db = 0; db < HD / 16; ++db) {
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      if (have[t])
-        va[db].d[t] = *reinterpret_cast<const uint2*>(v_cache + vbase[t] + (long)(db * 16 + lr) * page_size + lg * 4);
-      else
-        va[db].d[t] = make_uint2(0u, 0u);
-    }
-  }
-
-  // softmax update per column, then O^T += V^T . P^T
 #pragma unroll
   for (int c = 0; c < CB; ++c) {
     float p[2][4];
@@ -99,10 +104,13 @@ __device__ inline void attn_chunk(AttnState<HD, CB>& st, int k0, const bf16_t* _
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int key = k0 + t * 16 + lg * 4 + i;
-        const bool visible = have[t] && key <= st.pos[c] && key >= st.lo[c];
-        p[t][i] = visible ? s[t][c][i] * scale : -INFINITY;
-        mx = fmaxf(mx, p[t][i]);
+        float v = s[t][c][i] * scale_log2;
+        if (masked) {
+          const int key = k0 + t * 16 + lg * 4 + i;
+          if (!(kv.have[t] && key <= st.pos[c] && key >= st.lo[c])) v = -INFINITY;
+        }
+        p[t][i] = v;
+        mx = fmaxf(mx, v);
       }
     mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
     mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
@@ -114,12 +122,12 @@ __device__ inline void attn_chunk(AttnState<HD, CB>& st, int k0, const bf16_t* _
 #pragma unroll
         for (int i = 0; i < 4; ++i) p[t][i] = 0.f;
     } else {
-      alpha = expf(st.m[c] - m_new);
+      alpha = __builtin_amdgcn_exp2f(st.m[c] - m_new);
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-          p[t][i] = expf(p[t][i] - m_new);
+          p[t][i] = __builtin_amdgcn_exp2f(p[t][i] - m_new);
           sum += p[t][i];
         }
     }
@@ -136,13 +144,35 @@ __device__ inline void attn_chunk(AttnState<HD, CB>& st, int k0, const bf16_t* _
     for (int db = 0; db < HD / 16; ++db) {
       f32x4_t o = st.o[db][c];
       o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
-      st.o[db][c] = mfma16(va[db], pb, o);
+      st.o[db][c] = mfma16(kv.v[db], pb, o);
     }
   }
 }
 
+// Walk chunks c0 .. c1-1 (32 keys each) with the next chunk's loads in flight during the
+// current chunk's arithmetic.  Chunks from `first_unmasked` up to `last_unmasked` (inclusive)
+// are known to be fully visible to every column.
+template <int HD, int CB>
+__device__ inline void attn_walk(AttnState<HD, CB>& st, int c0, int c1, int first_unmasked, int last_unmasked,
+                                 const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
+                                 const int* __restrict__ bt, int table_width, int kv_len, int nkv, int g, int page_size,
+                                 long num_pages, float scale_log2, int lane) {
+  if (c0 >= c1) return;
+  KVChunk<HD> a, b;
+  attn_load<HD>(a, c0 * 32, k_cache, v_cache, bt, table_width, kv_len, nkv, g, page_size, num_pages, lane);
+  int c = c0;
+  while (true) {
+    if (c + 1 < c1) attn_load<HD>(b, (c + 1) * 32, k_cache, v_cache, bt, table_width, kv_len, nkv, g, page_size, num_pages, lane);
+    attn_compute<HD, CB>(st, a, c * 32, scale_log2, c < first_unmasked || c > last_unmasked, lane);
+    if (++c >= c1) break;
+    if (c + 1 < c1) attn_load<HD>(a, (c + 1) * 32, k_cache, v_cache, bt, table_width, kv_len, nkv, g, page_size, num_pages, lane);
+    attn_compute<HD, CB>(st, b, c * 32, scale_log2, c < first_unmasked || c > last_unmasked, lane);
+    if (++c >= c1) break;
+  }
+}
+
 // Load the query fragment of column block c: the lane's column is (token row `row`, head `head`),
-// or padding when valid is false.
+// or padding (zeros) when valid is false.
 template <int HD, int CB>
 __device__ inline void attn_load_q(AttnState<HD, CB>& st, int c, const bf16_t* __restrict__ q, long q_stride, long row,
                                    int head, bool valid, int lane) {

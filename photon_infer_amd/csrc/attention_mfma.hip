@@ -30,36 +30,44 @@ __global__ __launch_bounds__(256) void attention_tiles_kernel(
   attn_init(st);
   long rows[CB];
   int heads[CB];
-  int lo_w = 0x7fffffff, hi_w = -1;
+  bool valid[CB];
+  // over the wave's real columns: the first and last key any of them sees (the walk), and the
+  // keys all of them see (no masking needed there)
+  int lo_min = 0x7fffffff, lo_max = 0, pos_min = 0x7fffffff, pos_max = -1;
 #pragma unroll
   for (int c = 0; c < CB; ++c) {
     const int col = (wave * CB + c) * 16 + lr;
     const int tok = col / G;
-    const bool valid = tok < TQ && q0 + tok < q_len;
+    valid[c] = tok < TQ && q0 + tok < q_len;
     const int pos = kv_len - q_len + q0 + tok;
     rows[c] = qs + q0 + tok;
     heads[c] = g * G + col % G;
-    st.pos[c] = valid ? pos : -1;
-    st.lo[c] = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-    attn_load_q(st, c, q, q_stride, rows[c], heads[c], valid, lane);
-    if (valid) {
-      lo_w = min(lo_w, st.lo[c]);
-      hi_w = max(hi_w, pos);
+    // padding columns are computed on zeros, see everything and are never stored
+    st.pos[c] = valid[c] ? pos : 0x7fffffff;
+    st.lo[c] = (valid[c] && window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    attn_load_q(st, c, q, q_stride, rows[c], heads[c], valid[c], lane);
+    if (valid[c]) {
+      lo_min = min(lo_min, st.lo[c]);
+      lo_max = max(lo_max, st.lo[c]);
+      pos_min = min(pos_min, pos);
+      pos_max = max(pos_max, pos);
     }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
-    lo_w = min(lo_w, __shfl_xor(lo_w, off, 64));
-    hi_w = max(hi_w, __shfl_xor(hi_w, off, 64));
+    lo_min = min(lo_min, __shfl_xor(lo_min, off, 64));
+    lo_max = max(lo_max, __shfl_xor(lo_max, off, 64));
+    pos_min = min(pos_min, __shfl_xor(pos_min, off, 64));
+    pos_max = max(pos_max, __shfl_xor(pos_max, off, 64));
   }
-  if (hi_w < 0) return;   // no column of this wave is a real query
+  if (pos_max < 0) return;   // no column of this wave is a real query
 
-  for (int c = lo_w / 32; c <= hi_w / 32; ++c)
-    attn_chunk<HD, CB>(st, c * 32, k_cache, v_cache, bt, table_width, kv_len, nkv, g, page_size, num_pages, scale, lane);
+  attn_walk<HD, CB>(st, lo_min / 32, pos_max / 32 + 1, (lo_max + 31) / 32, (pos_min + 1) / 32 - 1, k_cache, v_cache, bt,
+                    table_width, kv_len, nkv, g, page_size, num_pages, scale * PI_LOG2E, lane);
 
 #pragma unroll
   for (int c = 0; c < CB; ++c) {
-    if (st.pos[c] < 0) continue;
+    if (!valid[c]) continue;
     const float inv = 1.0f / st.l[c];
     bf16_t* o = out + rows[c] * out_stride + (long)heads[c] * HD + lg * 4;
 #pragma unroll

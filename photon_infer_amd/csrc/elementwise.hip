@@ -138,8 +138,32 @@ extern "C" int pi_swiglu(void* out, const void* gu, int dtype, int T, int I, int
 // Cache layout: keys [page, kv_head, slot_in_page, head_dim]; values transposed,
 // [page, kv_head, head_dim, slot_in_page], so that the keys of one page are contiguous for a
 // fixed feature - the order in which the matrix-core attention kernels contract them.
-// angle = float(pos) * inv_freq[j]; pair j is (x[j], x[j + R/2]) or, interleaved,
-// (x[2j], x[2j+1]); (a, b) <- (a cos - b sin, a sin + b cos).  Dims >= R are copied.
+// Pair j is (x[j], x[j + R/2]) or, interleaved, (x[2j], x[2j+1]);
+// (a, b) <- (a cos - b sin, a sin + b cos) with cos / sin of the token's angle from the
+// step's table (rope_table_kernel below).  Dims >= R are copied.
+// table[t, j] = cos(angle), table[t, R/2 + j] = sin(angle), angle = float(pos[t]) * inv_freq[j]:
+// float32 product, full-range sine and cosine.  Made once per step and read by every layer.
+__global__ void rope_table_kernel(float* __restrict__ table, const int* __restrict__ positions,
+                                  const float* __restrict__ inv_freq, int T, int half) {
+  const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (long)T * half) return;
+  const long t = idx / half;
+  const int j = (int)(idx - t * half);
+  const float angle = (float)positions[t] * inv_freq[j];
+  float s, c;
+  sincosf(angle, &s, &c);
+  table[t * 2 * half + j] = c;
+  table[t * 2 * half + half + j] = s;
+}
+
+extern "C" int pi_rope_table(float* table, const int* positions, const float* inv_freq, int T, int half, hipStream_t stream) {
+  PI_REQUIRE(T >= 0 && half > 0 && table && positions && inv_freq, "rope_table: bad arguments T=%d half=%d", T, half);
+  if (T == 0) return 0;
+  const long total = (long)T * half;
+  hipLaunchKernelGGL(rope_table_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, stream, table, positions, inv_freq, T, half);
+  return pi_check_launch("rope_table");
+}
+
 // The source of q, k, v is either the projection's output in the compute dtype (q is rotated in
 // place) or, when `part` is given, the pieces of that projection still to be summed: float32
 // [splits, T, ncols] with q at column q_col, k at k_col, v at v_col; the rotated q then goes to
@@ -147,7 +171,7 @@ extern "C" int pi_swiglu(void* out, const void* gu, int dtype, int T, int I, int
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
                                      const T* __restrict__ v, long v_stride, const int* __restrict__ positions,
-                                     const int* __restrict__ req_of_token, const float* __restrict__ inv_freq,
+                                     const int* __restrict__ req_of_token, const float* __restrict__ table,
                                      int rotary_dim, int interleaved, int nh, int nkv_write, int nkv, int hd,
                                      T* __restrict__ k_cache, T* __restrict__ v_cache,
                                      const int* __restrict__ block_table, int table_width, int page_size,
@@ -194,7 +218,13 @@ __global__ void rope_kv_write_kernel(T* __restrict__ q, long q_stride, const T* 
     if (part) {
       val = 0.f;
       const float* p = part + t * ncols + col + d;
-      for (int s = 0; s < splits; ++s) val += p[s * part_stride];
+      for (int s0 = 0; s0 < splits; s0 += 8) {      // loads go out together, adds keep the split order
+        float tmp[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) tmp[u] = (s0 + u < splits) ? p[(s0 + u) * part_stride] : 0.f;
+#pragma unroll
+        for (int u = 0; u < 8; ++u) val += tmp[u];
+      }
     } else {
       val = to_float(src[d]);
     }
@@ -207,9 +237,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ q, long q_stride, const T* 
       const int i0 = interleaved ? 2 * j : j;
       const int i1 = interleaved ? 2 * j + 1 : j + half;
       const float a = head[i0], b = head[i1];
-      const float angle = (float)pos * inv_freq[j];
-      float s, c;
-      sincosf(angle, &s, &c);
+      const float c = table[t * rotary_dim + j], s = table[t * rotary_dim + half + j];
       dst[i0 * dst_stride] = from_float<T>(a * c - b * s);
       dst[i1 * dst_stride] = from_float<T>(a * s + b * c);
     }
@@ -220,14 +248,14 @@ __global__ void rope_kv_write_kernel(T* __restrict__ q, long q_stride, const T* 
 }
 
 extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
-                                int dtype, const int* positions, const int* req_of_token, const float* inv_freq,
+                                int dtype, const int* positions, const int* req_of_token, const float* table,
                                 int rotary_dim, int interleaved, int T, int nh, int nkv, int hd, int write_kv,
                                 void* k_cache, void* v_cache, const int* block_table, int table_width,
                                 int page_size, long num_pages, const float* part, int splits, int ncols, int q_col,
                                 int k_col, int v_col, hipStream_t stream) {
   PI_REQUIRE(T >= 0 && nh >= 0 && nkv >= 0 && hd > 0 && hd <= 256, "rope_kv_write: bad sizes T=%d heads=%d kv_heads=%d head_dim=%d", T, nh, nkv, hd);
   PI_REQUIRE(rotary_dim >= 0 && rotary_dim <= hd && rotary_dim % 2 == 0, "rope_kv_write: rotary_dim %d must be even and <= head_dim %d", rotary_dim, hd);
-  PI_REQUIRE(rotary_dim == 0 || inv_freq != nullptr, "rope_kv_write: rotation asked for without a frequency table");
+  PI_REQUIRE(rotary_dim == 0 || table != nullptr, "rope_kv_write: rotation asked for without a cos / sin table");
   PI_REQUIRE(part == nullptr || (splits >= 1 && ncols > 0), "rope_kv_write: bad split description");
   if (write_kv) {
     PI_REQUIRE((part || (k && v)) && k_cache && v_cache && block_table && req_of_token, "rope_kv_write: cache write asked for without k/v/cache/table");
@@ -241,12 +269,12 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
   const long part_stride = (long)T * ncols;
   if (dtype == PI_F32)
     hipLaunchKernelGGL(rope_kv_write_kernel<float>, grid, block, 0, stream, (float*)q, q_stride, (const float*)k, k_stride,
-                       (const float*)v, v_stride, positions, req_of_token, inv_freq, rotary_dim, interleaved, nh, nkv_write,
+                       (const float*)v, v_stride, positions, req_of_token, table, rotary_dim, interleaved, nh, nkv_write,
                        nkv, hd, (float*)k_cache, (float*)v_cache, block_table, table_width, page_size, num_pages, part,
                        splits, part_stride, ncols, q_col, k_col, v_col);
   else if (dtype == PI_BF16)
     hipLaunchKernelGGL(rope_kv_write_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)q, q_stride, (const bf16_t*)k, k_stride,
-                       (const bf16_t*)v, v_stride, positions, req_of_token, inv_freq, rotary_dim, interleaved, nh, nkv_write,
+                       (const bf16_t*)v, v_stride, positions, req_of_token, table, rotary_dim, interleaved, nh, nkv_write,
                        nkv, hd, (bf16_t*)k_cache, (bf16_t*)v_cache, block_table, table_width, page_size, num_pages, part,
                        splits, part_stride, ncols, q_col, k_col, v_col);
   else

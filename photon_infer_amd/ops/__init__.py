@@ -228,6 +228,33 @@ def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, hd: int
     return k_cache.shape[0]
 
 
+def rope_table(positions: torch.Tensor, inv_freq: torch.Tensor) -> torch.Tensor:
+    """float32 [T, 2 * half]: cos then sin of float32(position) * inv_freq[j], for every token."""
+    _gpu(positions, inv_freq)
+    T, half = positions.shape[0], inv_freq.numel()
+    _i32(positions, "positions")
+    if inv_freq.dtype != torch.float32 or not inv_freq.is_contiguous():
+        raise KernelError("rope: the frequency table must be contiguous float32")
+    table = torch.empty((T, 2 * half), dtype=torch.float32, device=positions.device)
+    _lib.call("core", "pi_rope_table", table.data_ptr(), positions.data_ptr(), inv_freq.data_ptr(), T, half, _stream())
+    return table
+
+
+def _rotary_args(rotary, positions, T):
+    """(table pointer, rotary_dim, interleaved) from ``rotary`` = (frequencies or table, R, interleaved)."""
+    if rotary is None:
+        return None, 0, False, None
+    src, rdim, inter = rotary
+    if src.dim() == 2:                       # already the step's cos / sin table
+        if src.shape != (T, rdim) or src.dtype != torch.float32 or not src.is_contiguous():
+            raise KernelError(f"rope: cos / sin table must be contiguous float32 [{T}, {rdim}]")
+        return src.data_ptr(), rdim, inter, src
+    if src.numel() != rdim // 2:
+        raise KernelError(f"rope: frequency table must be float32 [{rdim // 2}]")
+    table = rope_table(positions, src)
+    return table.data_ptr(), rdim, inter, table
+
+
 def qkv_projection(h: torch.Tensor, w_qkv: torch.Tensor, dtype: torch.dtype):
     """h @ w_qkv^T for the attention mixer: a tensor [T, N] in ``dtype``, or - when the
     product was split over k - its pieces (``fast.Partials``), which ``rope_kv_write`` sums
@@ -248,7 +275,8 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
                   block_table: Optional[torch.Tensor], page_size: int, pieces=None, write_kv: Optional[bool] = None) -> None:
     """Rotate q in place by each token's position; rotate k and store k, v into the pages.
 
-    ``rotary`` = (inv_freq float32 [R/2], R, interleaved) or None for no rotation.
+    ``rotary`` = (inv_freq float32 [R/2] or the step's cos / sin table [T, R], R, interleaved), or
+    None for no rotation.
     ``k``/``v`` None: queries only (the layer reads a cache that another one writes).
     ``pieces``: the q|k|v projection still split over k (``fast.Partials`` with columns
     [q heads | k heads | v heads]); then ``q`` is the output buffer for the rotated queries and
@@ -262,22 +290,20 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
     _i32(positions, "positions", T)
     if pieces is not None:
         write = bool(write_kv)
-        inv_freq, rdim, inter = (None, 0, False) if rotary is None else rotary
+        table_ptr, rdim, inter, _keep = _rotary_args(rotary, positions, T)
         q_size, kv_size = num_heads * head_dim, num_kv_heads * head_dim
         if pieces.M != T or pieces.N < q_size + (2 * kv_size if write else 0):
             raise KernelError(f"rope: pieces [{pieces.M}, {pieces.N}] do not hold q, k, v of {T} tokens")
         pages = _check_cache(k_cache, v_cache, num_kv_heads, head_dim, page_size, q.dtype) if write else 0
         _lib.call(
             "core", "pi_rope_kv_write", q.data_ptr(), _rows(q, "q"), None, 0, None, 0, _dt(q), positions.data_ptr(),
-            _ptr(req_of_token) if write else None, _ptr(inv_freq), rdim, int(bool(inter)), T, num_heads, num_kv_heads,
+            _ptr(req_of_token) if write else None, table_ptr, rdim, int(bool(inter)), T, num_heads, num_kv_heads,
             head_dim, int(write), _ptr(k_cache) if write else None, _ptr(v_cache) if write else None,
             _ptr(block_table) if write else None, block_table.shape[1] if write else 0, page_size if write else 0, pages,
             pieces.part.data_ptr(), pieces.splits, pieces.N, 0, q_size, q_size + kv_size, _stream())
         return
     write = k is not None
-    inv_freq, rdim, inter = (None, 0, False) if rotary is None else rotary
-    if inv_freq is not None and (inv_freq.dtype != torch.float32 or inv_freq.numel() != rdim // 2 or not inv_freq.is_contiguous()):
-        raise KernelError(f"rope: frequency table must be float32 [{rdim // 2}]")
+    table_ptr, rdim, inter, _keep = _rotary_args(rotary, positions, T)
     if not write and rdim == 0:
         return
     pages = 0
@@ -291,7 +317,7 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
     _lib.call(
         "core", "pi_rope_kv_write", q.data_ptr(), _rows(q, "q"), _ptr(k), _rows(k, "k") if write else 0, _ptr(v),
         _rows(v, "v") if write else 0, _dt(q), positions.data_ptr(), _ptr(req_of_token) if write else None,
-        _ptr(inv_freq), rdim, int(bool(inter)), T, num_heads, num_kv_heads, head_dim, int(write),
+        table_ptr, rdim, int(bool(inter)), T, num_heads, num_kv_heads, head_dim, int(write),
         _ptr(k_cache) if write else None, _ptr(v_cache) if write else None, _ptr(block_table) if write else None,
         block_table.shape[1] if write else 0, page_size if write else 0, pages, None, 0, 0, 0, 0, 0, _stream())
 

@@ -78,7 +78,7 @@ class PagedAttention(Mixer):
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
         T = h.shape[0]
         writes = self.own_kv and cache.writes
-        rotary = self.position.rotary_params() if self.position is not None else None
+        rotary = self.position.rotary_params(ctx) if self.position is not None else None
         fused_position = self.position is None or rotary is not None
         table = ctx.block_tables[cache.group]
         qkv = ops.qkv_projection(h, self.w_qkv, self.dtype) if fused_position else None

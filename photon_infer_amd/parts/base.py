@@ -83,6 +83,7 @@ class StepContext:
     decode_splits: int = 1                       # key ranges per request in split-K decode
     workspace: Any = None                        # engine-owned scratch tensors
     host_slots: Sequence[int] = ()
+    scratch: Dict[Any, Any] = field(default_factory=dict)   # what parts share within one step; emptied per step
 
 
 @dataclass
@@ -124,7 +125,7 @@ class PositionEncoding(Part):
     kernel; a scheme that is not a rotation returns None and implements ``apply``.
     """
 
-    def rotary_params(self):
+    def rotary_params(self, ctx=None):
         return None
 
     def apply(self, q: torch.Tensor, k: torch.Tensor, ctx: StepContext) -> None:

@@ -136,6 +136,7 @@ class DecoderModel:
         """Run the step's tokens through the run order; float32 logits [M, vocab] at
         ``ctx.logit_rows`` (None when no row is wanted)."""
         ops.reset_deferred()               # nothing of an earlier (failed) step may linger
+        ctx.scratch.clear()
         x = self.embedding.forward(ctx.token_ids)
         for i, entry in enumerate(self.spec.run_order):
             self.blocks[entry.layer].forward(x, ctx, caches[i])

@@ -66,8 +66,17 @@ class RotaryEmbedding(PositionEncoding):
                 dtype=torch.float32, device=device
             )
 
-    def rotary_params(self):
-        return self.inv_freq, self.rotary_dim, self.interleaved
+    def rotary_params(self, ctx=None):
+        """(frequencies, rotated width, pairing) - or, given the step's context, the step's
+        cos / sin table instead of the frequencies: every layer of a step rotates by the same
+        angles, so they are computed once."""
+        if ctx is None:
+            return self.inv_freq, self.rotary_dim, self.interleaved
+        table = ctx.scratch.get(("rope", id(self)))
+        if table is None:
+            from .. import ops
+            table = ctx.scratch[("rope", id(self))] = ops.rope_table(ctx.positions, self.inv_freq)
+        return table, self.rotary_dim, self.interleaved
 
 
 POSITION_ENCODINGS.register("rope", RotaryEmbedding)

@@ -75,7 +75,7 @@ def attention_ctx(q_lens: Sequence[int], kv_lens: Sequence[int], dtype) -> Simpl
     parts.update(plan.get("arrays", {}))
     views = _upload(parts, DEV)
     ctx = SimpleNamespace(T=int(sum(q_lens)), R=R, dtype=dtype, q_lens=list(q_lens), kv_lens=list(kv_lens),
-                          max_q_len=max(q_lens), max_kv_len=max(kv_lens), all_decode=all(n == 1 for n in q_lens),
+                          max_q_len=max(q_lens), max_kv_len=max(kv_lens), all_decode=all(n == 1 for n in q_lens), scratch={},
                           **{k: views[k] for k in ("positions", "req_of_token", "q_start", "kv_len")})
     ops.attach_attention_plan(ctx, plan, views)
     return ctx
