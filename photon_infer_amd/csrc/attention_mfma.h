@@ -112,8 +112,7 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv
         p[t][i] = v;
         mx = fmaxf(mx, v);
       }
-    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    mx = column_max(mx);
     const float m_new = fmaxf(st.m[c], mx);
     float alpha = 1.f, sum = 0.f;
     if (m_new == -INFINITY) {          // nothing visible yet in this column
@@ -131,8 +130,7 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv
           sum += p[t][i];
         }
     }
-    sum += __shfl_xor(sum, 16, 64);
-    sum += __shfl_xor(sum, 32, 64);
+    sum = column_sum(sum);
     st.l[c] = st.l[c] * alpha + sum;
     st.m[c] = m_new;
     Frag pb;

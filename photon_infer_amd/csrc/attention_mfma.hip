@@ -4,7 +4,9 @@
 // The step's tokens are cut into tiles of TQ consecutive tokens of one request (work list made
 // on the host).  A block of four waves handles one (tile, kv head): its 4 * CB * 16 query
 // columns are the tile's tokens times the heads of the kv group, so keys and values are read
-// once for the whole group.  Each wave walks the keys its own columns can see, 32 at a time,
+// once for the whole group.  Tiles are small (CB = 2) so that a prompt makes more blocks than
+// the chip has compute units and the short early tiles fill in around the long late ones.
+// Each wave walks the keys its own columns can see, 32 at a time,
 // with a running softmax per column; a token at absolute position p sees keys lo..p only
 // (lo = 0, or p - window + 1), whatever portion it arrived in.
 #include "attention_mfma.h"
@@ -18,7 +20,7 @@ __global__ __launch_bounds__(256) void attention_tiles_kernel(
     int window, long num_pages, int TQ) {
   const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
   const int lr = lane % 16, lg = lane / 16;
-  const int tile = blockIdx.x, g = blockIdx.y;
+  const int tile = gridDim.x - 1 - blockIdx.x, g = blockIdx.y;   // later tiles see more keys: start them first
   const int G = nh / nkv;
   const int r = tile_req[tile], q0 = tile_q0[tile];
   const int qs = q_start[r];
@@ -83,7 +85,7 @@ __global__ __launch_bounds__(256) void attention_tiles_kernel(
 // Tokens per tile for a head layout: the block's columns divided among the heads of a group.
 extern "C" int pi_attention_tile_rows(int nh, int nkv, int hd) {
   if (nkv <= 0 || nh <= 0 || nh % nkv) return 0;
-  const int cols = 4 * (hd <= 64 ? 4 : 2) * 16;
+  const int cols = 4 * 2 * 16;
   return cols / (nh / nkv);
 }
 
@@ -103,7 +105,7 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
 #define GO(H, C) hipLaunchKernelGGL((attention_tiles_kernel<H, C>), grid, block, 0, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, \
                                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, \
                                     kv_len, tile_req, tile_q0, nh, nkv, page_size, scale, window, num_pages, TQ)
-  if (hd == 64) GO(64, 4); else GO(128, 2);
+  if (hd == 64) GO(64, 2); else GO(128, 2);
 #undef GO
   return pi_check_launch("attention_prefill_mfma");
 }

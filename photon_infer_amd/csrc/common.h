@@ -33,11 +33,28 @@ __host__ __device__ inline uint16_t f32_to_bf16_bits(float f) {
   return (uint16_t)(u >> 16);
 }
 
+// on the device the conversion is one instruction (v_cvt_pk_bf16_f32, round to nearest even)
+typedef __bf16 pi_bf16x2_t __attribute__((ext_vector_type(2)));
+typedef float pi_f32x2_t __attribute__((ext_vector_type(2)));
+__host__ __device__ inline uint32_t f32x2_to_bf16x2_bits(float lo, float hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  pi_f32x2_t v = {lo, hi};
+  pi_bf16x2_t b = __builtin_convertvector(v, pi_bf16x2_t);
+  return *reinterpret_cast<uint32_t*>(&b);
+#else
+  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
+#endif
+}
+
 template <typename T> __host__ __device__ inline T from_float(float v);
 template <> __host__ __device__ inline float from_float<float>(float v) { return v; }
 template <> __host__ __device__ inline bf16_t from_float<bf16_t>(float v) {
   bf16_t r;
+#if defined(__HIP_DEVICE_COMPILE__)
+  r.bits = (uint16_t)(f32x2_to_bf16x2_bits(v, 0.f) & 0xffffu);
+#else
   r.bits = f32_to_bf16_bits(v);
+#endif
   return r;
 }
 
@@ -50,6 +67,30 @@ __device__ inline float wave_sum(float v) {
 __device__ inline float wave_max(float v) {
 #pragma unroll
   for (int off = PI_WAVE / 2; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, PI_WAVE));
+  return v;
+}
+
+// ---- reductions over the four lanes l, l+16, l+32, l+48 (one column of a matrix-core tile),
+// with the gfx950 row / half swaps instead of a trip through the LDS crossbar:
+// v_permlane16_swap exchanges the odd 16-lane rows of one register with the even rows of the
+// other, v_permlane32_swap the upper half of one with the lower half of the other; fed the
+// same value twice, the two results hold a lane's own value and its partner's.
+__device__ inline float column_max(float v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(a[0]), __uint_as_float(a[1]));
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = fmaxf(__uint_as_float(b[0]), __uint_as_float(b[1]));
+#endif
+  return v;
+}
+__device__ inline float column_sum(float v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  auto a = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(a[0]) + __uint_as_float(a[1]);
+  auto b = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  v = __uint_as_float(b[0]) + __uint_as_float(b[1]);
+#endif
   return v;
 }
 

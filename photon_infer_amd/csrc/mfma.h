@@ -36,6 +36,4 @@ __device__ inline Frag load_frag(const bf16_t* p) {
   return f;
 }
 
-__device__ inline uint32_t pack_bf16x2(float lo, float hi) {
-  return (uint32_t)f32_to_bf16_bits(lo) | ((uint32_t)f32_to_bf16_bits(hi) << 16);
-}
+__device__ inline uint32_t pack_bf16x2(float lo, float hi) { return f32x2_to_bf16x2_bits(lo, hi); }
