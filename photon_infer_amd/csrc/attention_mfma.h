@@ -55,27 +55,42 @@ __device__ inline void attn_init(AttnState<HD, CB>& st) {
 // Issue the loads of the 32 keys starting at k0 (a multiple of 32).  `bt` is the request's
 // block-table row, `kv_len` the number of keys its pages hold; page_size is a multiple of 16.
 // A tile whose page is missing (beyond the length, or given back by a window) loads zeros.
+// Page ids of a request, 64 consecutive block-table entries at a time in one register per lane
+// (lane i holds block base + i), read out with v_readlane: the loads of a chunk then depend on
+// no other load, and the table is read once per 64 pages instead of once per tile.
+struct PageCache {
+  int base = -(1 << 30);
+  int ids = -1;
+  __device__ inline int get(int blk, const int* __restrict__ bt, int table_width, int lane) {
+    if (blk < base || blk >= base + 64) {          // uniform: blk and base are the same in every lane
+      base = blk;
+      const int b = blk + lane;
+      ids = b < table_width ? bt[b] : -1;
+    }
+    return __builtin_amdgcn_readlane(ids, blk - base);
+  }
+};
+
+// The loads are unconditional (a missing tile reads page 0 and is zeroed by attn_compute), so
+// that the compiler can count them and wait for one chunk while the next is still in flight.
 template <int HD>
 __device__ inline void attn_load(KVChunk<HD>& kv, int k0, const bf16_t* __restrict__ k_cache,
-                                 const bf16_t* __restrict__ v_cache, const int* __restrict__ bt, int table_width,
-                                 int kv_len, int nkv, int g, int page_size, long num_pages, int lane) {
+                                 const bf16_t* __restrict__ v_cache, PageCache& pages, const int* __restrict__ bt,
+                                 int table_width, int kv_len, int nkv, int g, int page_size, long num_pages, int lane) {
   const int lr = lane % 16, lg = lane / 16;
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
     const int key0 = k0 + t * 16;
-    const int blk = key0 / page_size;
-    long page = -1;
-    if (key0 < kv_len && blk < table_width) page = bt[blk];
+    const int page = key0 < kv_len ? pages.get(key0 / page_size, bt, table_width, lane) : -1;
     kv.have[t] = page >= 0 && page < num_pages;
     const long pg = kv.have[t] ? page : 0;
     const int slot = key0 % page_size;
     const bf16_t* kp = k_cache + ((pg * nkv + g) * page_size + slot + lr) * HD + lg * 8;
     const bf16_t* vp = v_cache + (pg * nkv + g) * (long)page_size * HD + slot + (long)lr * page_size + lg * 4;
 #pragma unroll
-    for (int ks = 0; ks < HD / 32; ++ks) kv.k[t][ks] = kv.have[t] ? load_frag(kp + ks * 32) : zero_frag();
+    for (int ks = 0; ks < HD / 32; ++ks) kv.k[t][ks] = load_frag(kp + ks * 32);
 #pragma unroll
-    for (int db = 0; db < HD / 16; ++db)
-      kv.v[db].d[t] = kv.have[t] ? *reinterpret_cast<const uint2*>(vp + (long)db * 16 * page_size) : make_uint2(0u, 0u);
+    for (int db = 0; db < HD / 16; ++db) kv.v[db].d[t] = *reinterpret_cast<const uint2*>(vp + (long)db * 16 * page_size);
   }
 }
 
@@ -142,7 +157,12 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv
     for (int db = 0; db < HD / 16; ++db) {
       f32x4_t o = st.o[db][c];
       o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
-      st.o[db][c] = mfma16(kv.v[db], pb, o);
+      Frag va = kv.v[db];
+      if (masked) {   // a missing tile was read from page 0: its values must not meet even a zero weight
+        if (!kv.have[0]) va.d[0] = make_uint2(0u, 0u);
+        if (!kv.have[1]) va.d[1] = make_uint2(0u, 0u);
+      }
+      st.o[db][c] = mfma16(va, pb, o);
     }
   }
 }
@@ -157,13 +177,16 @@ __device__ inline void attn_walk(AttnState<HD, CB>& st, int c0, int c1, int firs
                                  long num_pages, float scale_log2, int lane) {
   if (c0 >= c1) return;
   KVChunk<HD> a, b;
-  attn_load<HD>(a, c0 * 32, k_cache, v_cache, bt, table_width, kv_len, nkv, g, page_size, num_pages, lane);
+  PageCache pages;
+  // the chunk after the last one is loaded too (its tiles lie beyond the keys and read page 0):
+  // one load per compute, no branch between them
+  attn_load<HD>(a, c0 * 32, k_cache, v_cache, pages, bt, table_width, kv_len, nkv, g, page_size, num_pages, lane);
   int c = c0;
   while (true) {
-    if (c + 1 < c1) attn_load<HD>(b, (c + 1) * 32, k_cache, v_cache, bt, table_width, kv_len, nkv, g, page_size, num_pages, lane);
+    attn_load<HD>(b, (c + 1 < c1 ? c + 1 : c) * 32, k_cache, v_cache, pages, bt, table_width, kv_len, nkv, g, page_size, num_pages, lane);
     attn_compute<HD, CB>(st, a, c * 32, scale_log2, c < first_unmasked || c > last_unmasked, lane);
     if (++c >= c1) break;
-    if (c + 1 < c1) attn_load<HD>(a, (c + 1) * 32, k_cache, v_cache, bt, table_width, kv_len, nkv, g, page_size, num_pages, lane);
+    attn_load<HD>(a, (c + 1 < c1 ? c + 1 : c) * 32, k_cache, v_cache, pages, bt, table_width, kv_len, nkv, g, page_size, num_pages, lane);
     attn_compute<HD, CB>(st, b, c * 32, scale_log2, c < first_unmasked || c > last_unmasked, lane);
     if (++c >= c1) break;
   }

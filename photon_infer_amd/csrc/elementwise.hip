@@ -169,19 +169,33 @@ extern "C" int pi_rope_table(float* table, const int* positions, const float* in
 // [splits, T, ncols] with q at column q_col, k at k_col, v at v_col; the rotated q then goes to
 // the q buffer, and nothing ever holds the unrotated values in reduced precision.
 template <typename T>
-__global__ void rope_kv_write_kernel(T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride,
-                                     const T* __restrict__ v, long v_stride, const int* __restrict__ positions,
-                                     const int* __restrict__ req_of_token, const float* __restrict__ table,
-                                     int rotary_dim, int interleaved, int nh, int nkv_write, int nkv, int hd,
-                                     T* __restrict__ k_cache, T* __restrict__ v_cache,
-                                     const int* __restrict__ block_table, int table_width, int page_size,
-                                     long num_pages, const float* __restrict__ part, int splits, long part_stride,
-                                     int ncols, int q_col, int k_col, int v_col) {
-  __shared__ float head[256];
+__device__ inline float rope_source(const T* __restrict__ src, const float* __restrict__ part, int splits, long part_stride, int i) {
+  if (!part) return to_float(src[i]);
+  float val = 0.f;
+  const float* p = part + i;
+  for (int s0 = 0; s0 < splits; s0 += 8) {      // loads go out together, adds keep the split order
+    float tmp[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) tmp[u] = (s0 + u < splits) ? p[(s0 + u) * part_stride] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) val += tmp[u];
+  }
+  return val;
+}
+
+// One wave per (token, head), four heads to a block; a lane owns whole pairs, so nothing is
+// shared between lanes and every load of a lane is independent of the others.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_write_kernel(
+    T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride, const T* __restrict__ v, long v_stride,
+    const int* __restrict__ positions, const int* __restrict__ req_of_token, const float* __restrict__ table,
+    int rotary_dim, int interleaved, int nh, int nkv_write, int nkv, int hd, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, const int* __restrict__ block_table, int table_width, int page_size, long num_pages,
+    const float* __restrict__ part, int splits, long part_stride, int ncols, int q_col, int k_col, int v_col) {
   const long t = blockIdx.x;
-  const int h = blockIdx.y;
-  const int lane = threadIdx.x;
-  const int pos = positions[t];
+  const int h = blockIdx.y * 4 + threadIdx.x / PI_WAVE;
+  const int lane = threadIdx.x % PI_WAVE;
+  if (h >= nh + 2 * nkv_write) return;
   T* dst;
   long dst_stride = 1;        // element stride of the destination (values are stored transposed)
   const T* src = nullptr;
@@ -195,6 +209,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ q, long q_stride, const T* 
     const int hh = h - nh;
     const bool is_v = hh >= nkv_write;
     const int g = is_v ? hh - nkv_write : hh;
+    const int pos = positions[t];
     const int r = req_of_token[t];
     const int blk = pos / page_size;
     if (blk >= table_width) return;
@@ -212,38 +227,22 @@ __global__ void rope_kv_write_kernel(T* __restrict__ q, long q_stride, const T* 
       dst = k_cache + ((page * nkv + g) * page_size + (pos % page_size)) * hd;
     }
   }
-  // the head's values in float32
-  for (int d = lane; d < hd; d += PI_WAVE) {
-    float val;
-    if (part) {
-      val = 0.f;
-      const float* p = part + t * ncols + col + d;
-      for (int s0 = 0; s0 < splits; s0 += 8) {      // loads go out together, adds keep the split order
-        float tmp[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) tmp[u] = (s0 + u < splits) ? p[(s0 + u) * part_stride] : 0.f;
-#pragma unroll
-        for (int u = 0; u < 8; ++u) val += tmp[u];
-      }
-    } else {
-      val = to_float(src[d]);
-    }
-    head[d] = val;
-  }
-  __syncthreads();
+  const float* pp = part ? part + t * ncols + col : nullptr;
   if (rotate) {
     const int half = rotary_dim / 2;
     for (int j = lane; j < half; j += PI_WAVE) {
       const int i0 = interleaved ? 2 * j : j;
       const int i1 = interleaved ? 2 * j + 1 : j + half;
-      const float a = head[i0], b = head[i1];
+      const float a = rope_source(src, pp, splits, part_stride, i0);
+      const float b = rope_source(src, pp, splits, part_stride, i1);
       const float c = table[t * rotary_dim + j], s = table[t * rotary_dim + half + j];
       dst[i0 * dst_stride] = from_float<T>(a * c - b * s);
       dst[i1 * dst_stride] = from_float<T>(a * s + b * c);
     }
-    for (int i = rotary_dim + lane; i < hd; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(head[i]);
-  } else {
-    for (int i = lane; i < hd; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(head[i]);
+    if (part || dst != src)
+      for (int i = rotary_dim + lane; i < hd; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(rope_source(src, pp, splits, part_stride, i));
+  } else if (part || dst != src) {
+    for (int i = lane; i < hd; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(rope_source(src, pp, splits, part_stride, i));
   }
 }
 
@@ -264,7 +263,7 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
   const int heads = nh + (write_kv ? 2 * nkv : 0);
   if (T == 0 || heads == 0) return 0;
   PI_REQUIRE(heads <= 65535, "rope_kv_write: too many heads (%d)", heads);
-  const dim3 grid(T, heads), block(PI_WAVE);
+  const dim3 grid(T, (heads + 3) / 4), block(256);
   const int nkv_write = write_kv ? nkv : 0;
   const long part_stride = (long)T * ncols;
   if (dtype == PI_F32)
