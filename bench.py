@@ -88,8 +88,10 @@ def prefill_flops(cfg, layers, T) -> float:
     return gemm + attn + head
 
 
-def time_decode(runner, batch, steps, warmup, context, seed=1):
-    """Median-free, plain timing: ``steps`` decode steps of ``batch`` requests that end at ``context``."""
+def time_decode(runner, batch, steps, warmup, context, seed=1, synthetic_cache=False):
+    """Plain timing of ``steps`` decode steps of ``batch`` requests that end at ``context``.
+    ``synthetic_cache``: instead of running the prompts through the model, reserve the pages
+    and fill the pools with random numbers (for profiles that should hold decode kernels only)."""
     import torch
 
     from photon_infer_amd.engine import StepEntry
@@ -101,9 +103,17 @@ def time_decode(runner, batch, steps, warmup, context, seed=1):
     rids = [f"d{batch}_{i}" for i in range(batch)]
     for rid in rids:
         runner.admit(rid)
+        if synthetic_cache:
+            runner.cache.reserve(rid, start_len)
+            runner.cache.commit(rid, start_len)
+            continue
         toks = torch.randint(0, vocab, (start_len,), generator=g).tolist()
         for i in range(0, start_len, 2048):
             runner.step([StepEntry(rid, toks[i:i + 2048])])
+    if synthetic_cache:
+        for lc in runner.layer_caches:
+            lc.k.normal_()
+            lc.v.normal_()
     last = torch.randint(0, vocab, (batch,), generator=g).tolist()
     temps, draws = [0.0] * batch, [0.0] * batch
 
@@ -159,6 +169,8 @@ def main() -> int:
                     help="fewer layers than the model has, if memory or time needs it (both numbers are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
+    ap.add_argument("--only", choices=["decode", "prefill"], default=None,
+                    help="run just the decode steps at --batch, or just the prefill (for profiling); prints a short line")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -170,10 +182,19 @@ def main() -> int:
         print("bench.py: no GPU available", file=sys.stderr)
         return 1
     elem = 2 if args.dtype == "bf16" else 4
-    big = 1 if args.no_points else 64
+    big = 1 if (args.no_points or args.only) else 64
     runner, cfg = make_runner(MODEL, args.layers, args.dtype, max(big, args.batch), (max(big, args.batch)) * (CONTEXT + 64))
     wbytes = weight_bytes(runner)
     kvb = kv_bytes_per_token(cfg, args.layers, elem)
+    if args.only == "prefill":
+        psec = time_prefill(runner, PREFILL_TOKENS, max(1, args.steps // 8))
+        print(json.dumps({"only": "prefill", "tokens": PREFILL_TOKENS, "ms": round(psec * 1e3, 3)}), flush=True)
+        return 0
+    if args.only == "decode":
+        sec, _ = time_decode(runner, args.batch, args.steps, args.warmup, CONTEXT, synthetic_cache=True)
+        print(json.dumps({"only": "decode", "batch": args.batch, "ms_per_step": round(sec * 1e3, 4),
+                          "cache": "random numbers, no prompt was run"}), flush=True)
+        return 0
 
     sec, mean_ctx = time_decode(runner, args.batch, args.steps, args.warmup, CONTEXT)
     value = args.batch / sec
