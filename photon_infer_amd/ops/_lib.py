@@ -23,7 +23,8 @@ _SIGNATURES = {
         "pi_sample": [P, P, L, P, P, I, I, P, L, P],
     },
     "bf16": {
-        "pi_gemm_mfma": [P, I, L, P, L, P, L, I, I, I, P],
+        "pi_gemm_mfma": [P, I, L, P, L, P, L, I, I, I, I, P],
+        "pi_gemm_mfma_pieces": [I, I],
         "pi_gemm_skinny": [P, I, L, P, L, P, L, I, I, I, I, P, L, P, P],
         "pi_splitk_reduce": [P, I, L, P, I, I, I, P],
         "pi_attention_tile_rows": [I, I, I],

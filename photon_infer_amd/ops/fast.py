@@ -26,9 +26,12 @@ EPI_BF16, EPI_F32, EPI_ACCUM, EPI_SWIGLU = 0, 1, 2, 3
 SKINNY_MAX_ROWS = 64
 ROWS_PER_BLOCK = 32            # weight rows per block of the skinny kernel
 TARGET_BLOCKS = 512            # blocks wanted in flight to keep HBM busy
-GEMM_PART_FLOATS = 4 << 20     # k-split partial sums of the skinny kernel
+GEMM_PART_FLOATS = 16 << 20    # workspace for the pieces of products split over k (64 MB)
+TILE_MAX_SPLITS = 4
 ATTN_PART_FLOATS = 4 << 20     # key-split partial results of decode attention
 MAX_DECODE_SPLITS = 32
+DECODE_WAVES_WANTED = 2048     # waves of the decode attention kernel that fill the chip
+DECODE_MIN_KEYS_PER_SPLIT = 128
 
 
 class _Workspace:
@@ -83,6 +86,15 @@ def _skinny_splits(M: int, N: int, K: int) -> int:
     return splits
 
 
+def _tile_splits(M: int, N: int, K: int) -> int:
+    """k-split of the tile kernel: only when its 128 x 128 tiles are too few to fill the chip."""
+    tiles = -(-M // 128) * -(-N // 128)
+    splits = min(TILE_MAX_SPLITS, TARGET_BLOCKS // max(1, tiles), K // 512)
+    while splits > 1 and splits * M * N > GEMM_PART_FLOATS:
+        splits -= 1
+    return max(1, splits)
+
+
 def _flush_pending() -> None:
     """The product scratch is about to be reused: finish whatever still lives in it."""
     for ptr in list(PENDING):
@@ -119,7 +131,18 @@ def gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc, may_defer=False) -> bool
     else:
         return False
     if M > SKINNY_MAX_ROWS:
-        _lib.call("bf16", "pi_gemm_mfma", out.data_ptr(), epilogue, ldc, a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K,
+        splits = _tile_splits(M, N, K) if may_defer else 1
+        if splits > 1:
+            # few output tiles, long k: split k so that every compute unit has work; the pieces
+            # stay in the workspace for the next norm of this stream
+            ws = workspace(a.device)
+            _flush_pending()
+            made = _lib.load("bf16").pi_gemm_mfma_pieces(K, splits)
+            _lib.call("bf16", "pi_gemm_mfma", ws.gemm_part.data_ptr(), EPI_F32, N, a.data_ptr(), lda, w.data_ptr(), ldw,
+                      M, N, K, splits, _stream())
+            PENDING[out.data_ptr()] = Partials(ws.gemm_part, made, M, N)
+            return True
+        _lib.call("bf16", "pi_gemm_mfma", out.data_ptr(), epilogue, ldc, a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K, 1,
                   _stream())
         return True
     pieces = _skinny(out.data_ptr(), epilogue, ldc, a, w, M, N, K, lda, ldw, _skinny_splits(M, N, K))
@@ -151,7 +174,7 @@ def gemm_swiglu(out, a, w, M, N, K, lda, ldw) -> bool:
         return False
     if M > SKINNY_MAX_ROWS:
         _lib.call("bf16", "pi_gemm_mfma", out.data_ptr(), EPI_SWIGLU, out.stride(0), a.data_ptr(), lda, w.data_ptr(), ldw,
-                  M, N, K, _stream())
+                  M, N, K, 1, _stream())
     else:
         _skinny(out.data_ptr(), EPI_SWIGLU, out.stride(0), a, w, M, N, K, lda, ldw, 1)
     return True
@@ -187,9 +210,9 @@ def _tiles(ctx, tile_rows: int, device):
 def decode_splits(R: int, num_kv_heads: int, max_kv_len: Optional[int] = None) -> int:
     """Key ranges per (request, kv head): enough waves to fill the chip, no more than the
     keys are worth."""
-    splits = max(1, min(MAX_DECODE_SPLITS, -(-2048 // (R * num_kv_heads))))
+    splits = max(1, min(MAX_DECODE_SPLITS, -(-DECODE_WAVES_WANTED // (R * num_kv_heads))))
     if max_kv_len is not None:
-        splits = min(splits, max(1, -(-max_kv_len // 128)))
+        splits = min(splits, max(1, -(-max_kv_len // DECODE_MIN_KEYS_PER_SPLIT)))
     return splits
 
 
