@@ -55,7 +55,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
   const long m0 = (long)tile_m * BM, n0 = (long)tile_n * BN;
 
   // global -> register staging: thread t moves 16-byte chunk (t % 8) of rows (t / 8) + 32 p
-  const int lrow = tid / 8, lchunk = tid % 8;
+  // (eight lanes move one row's 128 bytes; the next eight lanes take the row 8 further down, so
+  // that sixteen lanes land on 64 distinct LDS banks with rows 144 bytes apart)
+  const int lgrp = tid / 8, lchunk = tid % 8;
+  const int lrow = (lgrp / 16) * 16 + ((lgrp / 8) % 2) * 4 + (lgrp % 8) / 2 + 8 * (lgrp % 2);
   uint4 ra[4], rw[4];
   auto load_slab = [&](int k0) {
     const int k = k0 + lchunk * 8;
