@@ -31,8 +31,8 @@ class _Group:
     window: Optional[int]
     pool: PagePool
     table: np.ndarray                      # [max_slots, max_blocks] int32, -1 = no page
-    next_block: np.ndarray                 # [max_slots] blocks ever allocated (index of the next one)
-    first_block: np.ndarray                # [max_slots] first block still held
+    next_block: list                       # [max_slots] blocks ever allocated (index of the next one)
+    first_block: list                      # [max_slots] first block still held
 
 
 @dataclass
@@ -58,7 +58,7 @@ class CacheManager:
             raise CacheError(f"{len(windows)} cache groups but {len(counts)} pool sizes")
         self.groups: List[_Group] = [
             _Group(w, PagePool(n), np.full((self.max_slots, self.max_blocks), -1, np.int32),
-                   np.zeros(self.max_slots, np.int64), np.zeros(self.max_slots, np.int64))
+                   [0] * self.max_slots, [0] * self.max_slots)
             for w, n in zip(windows, counts)
         ]
         self._requests: Dict[Hashable, _Request] = {}
@@ -97,7 +97,10 @@ class CacheManager:
         r = self._requests.get(rid) if rid is not None else None
         target = (r.length if r else 0) + new_tokens
         blocks = -(-target // self.page_size)
-        return [max(0, blocks - (int(g.next_block[r.slot]) if r else 0)) for g in self.groups]
+        if r is None:
+            return [blocks] * len(self.groups)
+        slot = r.slot
+        return [max(0, blocks - g.next_block[slot]) for g in self.groups]
 
     def can_reserve(self, rid: Optional[Hashable], new_tokens: int, held_back: Sequence[int] | None = None) -> bool:
         """Whether ``reserve`` would succeed; ``held_back[g]`` pages of group g count as taken."""
@@ -188,7 +191,7 @@ class CacheManager:
         if not len(slots):
             return 0
         idx = np.asarray(slots, dtype=np.int64)
-        return int(max(int(g.next_block[idx].max()) for g in self.groups)) if self.groups else 0
+        return max(max(g.next_block[int(i)] for i in idx) for g in self.groups) if self.groups else 0
 
     # ------------------------------------------------------------------ checks and numbers
     def check_invariants(self) -> None:

@@ -11,7 +11,7 @@
 #include "attention_mfma.h"
 
 template <int HD>
-__global__ __launch_bounds__(64) void attention_decode_kernel(
+__global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2 : 1))) void attention_decode_kernel(
     bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q, long q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ q_start, const int* __restrict__ kv_len_of, int nh, int nkv, int page_size,
@@ -40,6 +40,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
   const int c1 = min(last_chunk + 1, c0 + per);
   attn_walk<HD, 1>(st, c0, c1, (lo + 31) / 32, (p + 1) / 32 - 1, k_cache, v_cache, bt, table_width, kv_len, nkv, g,
                    page_size, num_pages, scale * PI_LOG2E, lane);
+  attn_finish(st);
 
   const int head = g * G + lr;
   if (splits == 1) {
@@ -64,7 +65,7 @@ __global__ __launch_bounds__(64) void attention_decode_kernel(
     for (int db = 0; db < HD / 16; ++db)
       *reinterpret_cast<f32x4_t*>(mine + db * 16 + lg * 4) = st.o[db][0];
     if (lg == 0) {
-      mine[HD] = st.m[0];
+      mine[HD] = st.m[0] * (scale * PI_LOG2E);   // base-2 scale; -inf stays -inf
       mine[HD + 1] = st.l[0];
     }
   }

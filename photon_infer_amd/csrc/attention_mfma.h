@@ -13,10 +13,9 @@
 // 8-byte loads.  Running maximum, running sum and the rescaling factor belong to a column,
 // i.e. to lane % 16, replicated over the four lane groups.
 //
-// Scores, softmax and both accumulations are float32.  The exponential is taken in base 2
-// (scores are scaled by scale * log2(e) once, then v_exp_f32), so the running maximum is kept
-// in that scale too.  P is rounded to bfloat16 for the second product; the sum of P is taken
-// before rounding.
+// Scores, softmax and both accumulations are float32.  The exponential is taken in base 2:
+// a weight is 2^((score - reference) * scale * log2(e)), one fused multiply-add and v_exp_f32.
+// P is rounded to bfloat16 for the second product; the sum of P is taken before rounding.
 //
 // The keys and values of a chunk are loaded into registers by attn_load and consumed by
 // attn_compute, so a caller can have the next chunk's loads in flight while it computes.
@@ -29,7 +28,8 @@ template <int HD, int CB>
 struct AttnState {
   Frag q[CB][HD / 32];
   f32x4_t o[HD / 16][CB];
-  float m[CB], l[CB];   // running maximum (base-2 scale) and running sum per column
+  float m[CB];          // reference score of the column (raw units, see attn_compute)
+  float l[CB];          // this lane's share of the column's sum of weights: attn_finish adds the four shares
   int pos[CB];          // last visible key of the column
   int lo[CB];           // first visible key of the column
 };
@@ -52,53 +52,104 @@ __device__ inline void attn_init(AttnState<HD, CB>& st) {
   }
 }
 
-// Issue the loads of the 32 keys starting at k0 (a multiple of 32).  `bt` is the request's
-// block-table row, `kv_len` the number of keys its pages hold; page_size is a multiple of 16.
-// A tile whose page is missing (beyond the length, or given back by a window) loads zeros.
-// Page ids of a request, 64 consecutive block-table entries at a time in one register per lane
-// (lane i holds block base + i), read out with v_readlane: the loads of a chunk then depend on
-// no other load, and the table is read once per 64 pages instead of once per tile.
-struct PageCache {
-  int base = -(1 << 30);
-  int ids = -1;
-  __device__ inline int get(int blk, const int* __restrict__ bt, int table_width, int lane) {
-    if (blk < base || blk >= base + 64) {          // uniform: blk and base are the same in every lane
-      base = blk;
-      const int b = blk + lane;
-      ids = b < table_width ? bt[b] : -1;
+// After the last chunk: the column's sum of weights from the four lanes that share it.
+template <int HD, int CB>
+__device__ inline void attn_finish(AttnState<HD, CB>& st) {
+#pragma unroll
+  for (int c = 0; c < CB; ++c) st.l[c] = column_sum(st.l[c]);
+}
+
+// Where the two key tiles of a chunk lie: page id (-1: none) and first slot in the page.  The
+// same in every lane, so they live in scalar registers and are fetched by scalar loads, which
+// the vector memory counter does not see: a table lookup never makes a wave wait for the keys
+// and values that are still in flight.
+struct ChunkPages {
+  int page[2];
+  int slot[2];
+};
+
+// Walks a request's block-table row tile by tile (16 keys; page_size is a multiple of 16).
+struct PageCursor {
+  typedef const int __attribute__((address_space(4)))* ScalarIntPtr;   // constant address space: scalar loads
+  ScalarIntPtr bt;    // block-table row, uniform
+  int table_width, kv_len, page_size;
+  int key, blk, slot; // next tile
+  __device__ inline void start(const int* row, int width, int len, int psize, int key0) {
+    const uint64_t v = reinterpret_cast<uint64_t>(row);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+    bt = (ScalarIntPtr)((static_cast<uint64_t>(hi) << 32) | lo);
+    table_width = __builtin_amdgcn_readfirstlane(width);
+    kv_len = __builtin_amdgcn_readfirstlane(len);
+    page_size = __builtin_amdgcn_readfirstlane(psize);
+    key = __builtin_amdgcn_readfirstlane(key0);
+    blk = __builtin_amdgcn_readfirstlane(key0 / psize);
+    slot = key - blk * page_size;
+  }
+  // A tile beyond the keys or beyond the table has no page.
+  __device__ inline ChunkPages next() {
+    ChunkPages cp;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      const bool ok = key < kv_len && blk < table_width;
+      const int id = bt[ok ? blk : 0];
+      cp.page[t] = ok ? id : -1;
+      cp.slot[t] = slot;
+      key += 16;
+      slot += 16;
+      if (slot >= page_size) { slot = 0; ++blk; }
     }
-    return __builtin_amdgcn_readlane(ids, blk - base);
+    return cp;
   }
 };
 
-// The loads are unconditional (a missing tile reads page 0 and is zeroed by attn_compute), so
-// that the compiler can count them and wait for one chunk while the next is still in flight.
+// What a lane adds to a tile's base address: fixed for a whole walk (bytes, 32 bits).
 template <int HD>
-__device__ inline void attn_load(KVChunk<HD>& kv, int k0, const bf16_t* __restrict__ k_cache,
-                                 const bf16_t* __restrict__ v_cache, PageCache& pages, const int* __restrict__ bt,
-                                 int table_width, int kv_len, int nkv, int g, int page_size, long num_pages, int lane) {
-  const int lr = lane % 16, lg = lane / 16;
+struct KVLaneOffsets {
+  uint32_t k;              // key row lane % 16, features (lane / 16) * 8 ..
+  uint32_t v[HD / 16];     // value row db * 16 + lane % 16, keys (lane / 16) * 4 ..
+  __device__ inline void set(int page_size, int lane) {
+    const int lr = lane % 16, lg = lane / 16;
+    k = (uint32_t)(lr * HD + lg * 8) * 2u;
+#pragma unroll
+    for (int db = 0; db < HD / 16; ++db) v[db] = (uint32_t)((db * 16 + lr) * page_size + lg * 4) * 2u;
+  }
+};
+
+// Issue the loads of a chunk of 32 keys.  The loads are unconditional (a missing tile reads
+// page 0 and is zeroed by attn_compute), so that the compiler can count them and wait for one
+// chunk while the next is still in flight.  A tile's base address is the same in every lane
+// (scalar arithmetic); the lane's part is a 32-bit offset.
+template <int HD>
+__device__ inline void attn_load(KVChunk<HD>& kv, const ChunkPages& cp, const bf16_t* __restrict__ k_cache,
+                                 const bf16_t* __restrict__ v_cache, const KVLaneOffsets<HD>& off, int nkv, int g,
+                                 int page_size, int num_pages) {
+  const long page_elems = (long)nkv * page_size * HD;
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
-    const int key0 = k0 + t * 16;
-    const int page = key0 < kv_len ? pages.get(key0 / page_size, bt, table_width, lane) : -1;
-    kv.have[t] = page >= 0 && page < num_pages;
-    const long pg = kv.have[t] ? page : 0;
-    const int slot = key0 % page_size;
-    const bf16_t* kp = k_cache + ((pg * nkv + g) * page_size + slot + lr) * HD + lg * 8;
-    const bf16_t* vp = v_cache + (pg * nkv + g) * (long)page_size * HD + slot + (long)lr * page_size + lg * 4;
+    kv.have[t] = cp.page[t] >= 0 && cp.page[t] < num_pages;
+    const long pg = kv.have[t] ? cp.page[t] : 0;
+    const char* kp = reinterpret_cast<const char*>(k_cache + pg * page_elems + (long)(g * page_size + cp.slot[t]) * HD);
+    const char* vp = reinterpret_cast<const char*>(v_cache + pg * page_elems + (long)g * page_size * HD + cp.slot[t]);
 #pragma unroll
-    for (int ks = 0; ks < HD / 32; ++ks) kv.k[t][ks] = load_frag(kp + ks * 32);
+    for (int ks = 0; ks < HD / 32; ++ks) kv.k[t][ks].q = *reinterpret_cast<const uint4*>(kp + off.k + ks * 64);
 #pragma unroll
-    for (int db = 0; db < HD / 16; ++db) kv.v[db].d[t] = *reinterpret_cast<const uint2*>(vp + (long)db * 16 * page_size);
+    for (int db = 0; db < HD / 16; ++db) kv.v[db].d[t] = *reinterpret_cast<const uint2*>(vp + off.v[db]);
   }
 }
 
-// Fold one loaded chunk into the state.  `masked`: some key of the chunk may be invisible to
-// some column (causal edge, window edge, missing tile); otherwise the per-key tests are skipped.
-template <int HD, int CB>
-__device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv, int k0, float scale_log2, bool masked,
-                                    int lane) {
+// How far (in powers of two) a column's scores may rise above its reference before the
+// reference is moved and the column rescaled.  Weights then stay below 2^8, sums far inside
+// float32; the reference cancels in the final division, so the result is the same softmax.
+#define PI_RESCALE_SLACK 8.0f
+
+// Fold one loaded chunk into the state.  MASKED: some key of the chunk may be invisible to
+// some column (causal edge, window edge, missing tile); otherwise the per-key tests are left out.
+// st.m is a column's reference score (raw, before the softmax scale): at least the largest
+// score seen minus the slack.  Moving it costs a pass over the accumulators, so it only moves
+// when some column of the wave needs it.
+template <int HD, int CB, bool MASKED>
+__device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv, int k0, float scale_log2, int lane) {
   const int lg = lane / 16;
   f32x4_t s[2][CB];
 #pragma unroll
@@ -110,44 +161,48 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv
       for (int ks = 0; ks < HD / 32; ++ks) acc = mfma16(kv.k[t][ks], st.q[c][ks], acc);
       s[t][c] = acc;
     }
+  const float slack = PI_RESCALE_SLACK / scale_log2;
 
 #pragma unroll
   for (int c = 0; c < CB; ++c) {
-    float p[2][4];
     float mx = -INFINITY;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float v = s[t][c][i] * scale_log2;
-        if (masked) {
+        if (MASKED) {
           const int key = k0 + t * 16 + lg * 4 + i;
-          if (!(kv.have[t] && key <= st.pos[c] && key >= st.lo[c])) v = -INFINITY;
+          if (!(kv.have[t] && key <= st.pos[c] && key >= st.lo[c])) s[t][c][i] = -INFINITY;
         }
-        p[t][i] = v;
-        mx = fmaxf(mx, v);
+        mx = fmaxf(mx, s[t][c][i]);
       }
-    mx = column_max(mx);
-    const float m_new = fmaxf(st.m[c], mx);
-    float alpha = 1.f, sum = 0.f;
-    if (m_new == -INFINITY) {          // nothing visible yet in this column
+    // the cheap test first: does any lane hold a score that far above its column's reference?
+    float m_ref = st.m[c];
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m_ref + slack) != 0, 0)) {   // also at the first visible key: m_ref is -inf then
+      mx = column_max(mx);
+      const bool move = mx > m_ref + slack;
+      const float alpha = move ? __builtin_amdgcn_exp2f((m_ref - mx) * scale_log2) : 1.f;
+      m_ref = move ? mx : m_ref;
+      st.m[c] = m_ref;
+      st.l[c] *= alpha;
 #pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) p[t][i] = 0.f;
-    } else {
-      alpha = __builtin_amdgcn_exp2f(st.m[c] - m_new);
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          p[t][i] = __builtin_amdgcn_exp2f(p[t][i] - m_new);
-          sum += p[t][i];
-        }
+      for (int db = 0; db < HD / 16; ++db) {
+        st.o[db][c][0] *= alpha; st.o[db][c][1] *= alpha; st.o[db][c][2] *= alpha; st.o[db][c][3] *= alpha;
+      }
     }
-    sum = column_sum(sum);
-    st.l[c] = st.l[c] * alpha + sum;
-    st.m[c] = m_new;
+    // weights 2^((score - reference) * scale); a column that has seen nothing yet has only -inf scores
+    float mc = m_ref * scale_log2;
+    if (MASKED) mc = (m_ref == -INFINITY) ? 0.f : mc;
+    float p[2][4];
+    float sum = 0.f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        p[t][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][c][i], scale_log2, -mc));
+        sum += p[t][i];
+      }
+    st.l[c] += sum;
     Frag pb;
     pb.q.x = pack_bf16x2(p[0][0], p[0][1]);
     pb.q.y = pack_bf16x2(p[0][2], p[0][3]);
@@ -155,16 +210,21 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv
     pb.q.w = pack_bf16x2(p[1][2], p[1][3]);
 #pragma unroll
     for (int db = 0; db < HD / 16; ++db) {
-      f32x4_t o = st.o[db][c];
-      o[0] *= alpha; o[1] *= alpha; o[2] *= alpha; o[3] *= alpha;
       Frag va = kv.v[db];
-      if (masked) {   // a missing tile was read from page 0: its values must not meet even a zero weight
+      if (MASKED) {   // a missing tile was read from page 0: its values must not meet even a zero weight
         if (!kv.have[0]) va.d[0] = make_uint2(0u, 0u);
         if (!kv.have[1]) va.d[1] = make_uint2(0u, 0u);
       }
-      st.o[db][c] = mfma16(va, pb, o);
+      st.o[db][c] = mfma16(va, pb, st.o[db][c]);
     }
   }
+}
+
+template <int HD, int CB>
+__device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv, int k0, float scale_log2, bool masked,
+                                    int lane) {
+  if (masked) attn_compute<HD, CB, true>(st, kv, k0, scale_log2, lane);
+  else attn_compute<HD, CB, false>(st, kv, k0, scale_log2, lane);
 }
 
 // Walk chunks c0 .. c1-1 (32 keys each) with the next chunk's loads in flight during the
@@ -174,21 +234,34 @@ template <int HD, int CB>
 __device__ inline void attn_walk(AttnState<HD, CB>& st, int c0, int c1, int first_unmasked, int last_unmasked,
                                  const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                                  const int* __restrict__ bt, int table_width, int kv_len, int nkv, int g, int page_size,
-                                 long num_pages, float scale_log2, int lane) {
+                                 long num_pages_l, float scale_log2, int lane) {
+  // the range is the same in every lane; saying so keeps the loop's branches scalar, and a
+  // divergent break would make the compiler wait for every load at the loop's head
+  c0 = __builtin_amdgcn_readfirstlane(c0);
+  c1 = __builtin_amdgcn_readfirstlane(c1);
+  first_unmasked = __builtin_amdgcn_readfirstlane(first_unmasked);
+  last_unmasked = __builtin_amdgcn_readfirstlane(last_unmasked);
   if (c0 >= c1) return;
   KVChunk<HD> a, b;
-  PageCache pages;
-  // the chunk after the last one is loaded too (its tiles lie beyond the keys and read page 0):
-  // one load per compute, no branch between them
-  attn_load<HD>(a, c0 * 32, k_cache, v_cache, pages, bt, table_width, kv_len, nkv, g, page_size, num_pages, lane);
-  int c = c0;
-  while (true) {
-    attn_load<HD>(b, (c + 1 < c1 ? c + 1 : c) * 32, k_cache, v_cache, pages, bt, table_width, kv_len, nkv, g, page_size, num_pages, lane);
+  KVLaneOffsets<HD> off;
+  off.set(page_size, lane);
+  const int num_pages = (int)(num_pages_l < 0x7fffffffL ? num_pages_l : 0x7fffffffL);
+  PageCursor cur;
+  cur.start(bt, table_width, kv_len, page_size, c0 * 32);
+  // Page ids run two chunks ahead, keys and values one chunk ahead of the arithmetic.  Two
+  // chunks per turn with fixed roles for the two buffers and no way out of the loop between
+  // them: the loads of one buffer are then always the youngest in flight when the other is
+  // consumed, which lets the compiler wait by count.  Up to two chunks beyond the range are
+  // loaded and never used.
+  ChunkPages pa = cur.next(), pb = cur.next();
+  attn_load<HD>(a, pa, k_cache, v_cache, off, nkv, g, page_size, num_pages);
+  for (int c = c0; c < c1; c += 2) {
+    pa = cur.next();
+    attn_load<HD>(b, pb, k_cache, v_cache, off, nkv, g, page_size, num_pages);
     attn_compute<HD, CB>(st, a, c * 32, scale_log2, c < first_unmasked || c > last_unmasked, lane);
-    if (++c >= c1) break;
-    attn_load<HD>(a, (c + 1 < c1 ? c + 1 : c) * 32, k_cache, v_cache, pages, bt, table_width, kv_len, nkv, g, page_size, num_pages, lane);
-    attn_compute<HD, CB>(st, b, c * 32, scale_log2, c < first_unmasked || c > last_unmasked, lane);
-    if (++c >= c1) break;
+    pb = cur.next();
+    attn_load<HD>(a, pa, k_cache, v_cache, off, nkv, g, page_size, num_pages);
+    if (c + 1 < c1) attn_compute<HD, CB>(st, b, (c + 1) * 32, scale_log2, c + 1 < first_unmasked || c + 1 > last_unmasked, lane);
   }
 }
 

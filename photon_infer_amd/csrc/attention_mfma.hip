@@ -12,7 +12,7 @@
 #include "attention_mfma.h"
 
 template <int HD, int CB>
-__global__ __launch_bounds__(256) void attention_tiles_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2 : 1))) void attention_tiles_kernel(
     bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q, long q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ q_start, const int* __restrict__ kv_len_of,
@@ -66,6 +66,7 @@ __global__ __launch_bounds__(256) void attention_tiles_kernel(
 
   attn_walk<HD, CB>(st, lo_min / 32, pos_max / 32 + 1, (lo_max + 31) / 32, (pos_min + 1) / 32 - 1, k_cache, v_cache, bt,
                     table_width, kv_len, nkv, g, page_size, num_pages, scale * PI_LOG2E, lane);
+  attn_finish(st);
 
 #pragma unroll
   for (int c = 0; c < CB; ++c) {

@@ -18,15 +18,19 @@ from .step import ModelRunner, StepEntry
 
 
 class ContinuousBatchEngine:
-    def __init__(self, model_dir: str, options: Optional[EngineOptions] = None, **option_fields):
+    def __init__(self, model_dir: Optional[str], options: Optional[EngineOptions] = None, *,
+                 runner: Optional[ModelRunner] = None, **option_fields):
         """``ContinuousBatchEngine(model_dir, dtype="bfloat16", max_batch=64, ...)``: any field
-        of EngineOptions may be given by keyword."""
-        if options is None:
+        of EngineOptions may be given by keyword.  ``runner``: use a ModelRunner that already
+        holds the model (then ``model_dir`` is None and the runner's options apply)."""
+        if runner is not None:
+            options = runner.options
+        elif options is None:
             options = EngineOptions(**option_fields)
         elif option_fields:
             raise RequestError("give either an EngineOptions object or option fields, not both")
         self.options = options
-        self.runner = ModelRunner(model_dir, options)
+        self.runner = runner if runner is not None else ModelRunner(model_dir, options)
         self.scheduler = ContinuousBatchScheduler(
             self.runner.cache, options.max_batch, options.max_step_tokens, options.chunk_size,
             self.runner.max_model_len, owner=self.runner)

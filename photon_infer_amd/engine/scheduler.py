@@ -47,6 +47,7 @@ class InferenceRequest:
         self.request_id = request_id
         self.prompt = prompt
         self.prompt_tokens: List[int] = [int(t) for t in prompt_tokens]
+        self._prompt_len = len(self.prompt_tokens)
         self.params = params
         self.state = RequestState.WAITING
         self.num_computed_tokens = 0
@@ -69,14 +70,14 @@ class InferenceRequest:
         return len(self.generated_tokens)
 
     def total_tokens(self) -> int:
-        return len(self.prompt_tokens) + len(self.generated_tokens)
+        return self._prompt_len + len(self.generated_tokens)
 
     def all_tokens(self) -> List[int]:
         return self.prompt_tokens + self.generated_tokens
 
     def remaining(self) -> int:
         """Known tokens that have not been fed through the model yet (>= 1 while running)."""
-        return self.total_tokens() - self.num_computed_tokens
+        return self._prompt_len + len(self.generated_tokens) - self.num_computed_tokens
 
     # ---- phases (a request that was preempted is a prompt again)
     def is_finished(self) -> bool:
@@ -86,7 +87,8 @@ class InferenceRequest:
         return self.remaining() > 1 or not self.generated_tokens
 
     def is_decode(self) -> bool:
-        return not self.is_finished() and not self.is_prefill()
+        return (self.state is not RequestState.FINISHED and bool(self.generated_tokens)
+                and self._prompt_len + len(self.generated_tokens) - self.num_computed_tokens == 1)
 
     def next_tokens(self, n: int) -> List[int]:
         c = self.num_computed_tokens
@@ -216,7 +218,10 @@ class ContinuousBatchScheduler:
 
     # ------------------------------------------------------------------ one step's decisions
     def _fits(self, need: Sequence[int], held: Sequence[int]) -> bool:
-        return all(n <= self.cache.free_pages(g) - held[g] for g, n in enumerate(need))
+        for g, n in enumerate(need):
+            if n and n > self.cache.free_pages(g) - held[g]:
+                return False
+        return True
 
     def _preempt(self, victim: InferenceRequest, batch: ScheduledBatch, held: List[int]) -> None:
         for i, (r, n) in enumerate(batch.items):
@@ -239,7 +244,8 @@ class ContinuousBatchScheduler:
         held = [0] * len(self.cache.groups)
 
         # Phase 1: running requests; those with a single token to feed first
-        order = [r for r in self.running if r.is_decode()] + [r for r in self.running if not r.is_decode()]
+        decoding = [r.is_decode() for r in self.running]
+        order = [r for r, d in zip(self.running, decoding) if d] + [r for r, d in zip(self.running, decoding) if not d]
         for req in order:
             if req not in self.running:      # preempted while serving an earlier one
                 continue
