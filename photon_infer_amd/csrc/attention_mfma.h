@@ -132,7 +132,7 @@ __device__ inline void attn_load(KVChunk<HD>& kv, const ChunkPages& cp, const bf
     const char* kp = reinterpret_cast<const char*>(k_cache + pg * page_elems + (long)(g * page_size + cp.slot[t]) * HD);
     const char* vp = reinterpret_cast<const char*>(v_cache + pg * page_elems + (long)g * page_size * HD + cp.slot[t]);
 #pragma unroll
-    for (int ks = 0; ks < HD / 32; ++ks) kv.k[t][ks].q = *reinterpret_cast<const uint4*>(kp + off.k + ks * 64);
+    for (int ks = 0; ks < HD / 32; ++ks) kv.k[t][ks].n = *reinterpret_cast<const u32x4_t*>(kp + off.k + ks * 64);
 #pragma unroll
     for (int db = 0; db < HD / 16; ++db) kv.v[db].d[t] = *reinterpret_cast<const uint2*>(vp + off.v[db]);
   }
@@ -273,5 +273,6 @@ __device__ inline void attn_load_q(AttnState<HD, CB>& st, int c, const bf16_t* _
   const int lg = lane / 16;
 #pragma unroll
   for (int ks = 0; ks < HD / 32; ++ks)
-    st.q[c][ks] = valid ? load_frag(q + row * q_stride + (long)head * HD + ks * 32 + lg * 8) : zero_frag();
+    st.q[c][ks].n = valid ? *reinterpret_cast<const u32x4_t*>(q + row * q_stride + (long)head * HD + ks * 32 + lg * 8)
+                          : u32x4_t{0u, 0u, 0u, 0u};
 }

@@ -2,83 +2,147 @@
 // cache, bfloat16 on the matrix cores.
 //
 // The step's tokens are cut into tiles of TQ consecutive tokens of one request (work list made
-// on the host).  A block of four waves handles one (tile, kv head): its 4 * CB * 16 query
-// columns are the tile's tokens times the heads of the kv group, so keys and values are read
-// once for the whole group.  Tiles are small (CB = 2) so that a prompt makes more blocks than
-// the chip has compute units and the short early tiles fill in around the long late ones.
-// Each wave walks the keys its own columns can see, 32 at a time,
-// with a running softmax per column; a token at absolute position p sees keys lo..p only
-// (lo = 0, or p - window + 1), whatever portion it arrived in.
+// on the host).  A block of four waves handles one (tile, kv head) at a time: its 4 * CB * 16
+// query columns are the tile's tokens times the heads of the kv group, so keys and values are
+// read once for the whole group.  The block walks the keys 128 at a time: each wave fetches 32
+// of them from the pages into registers while all four compute on the previous 128, which
+// they share through LDS (stored in the very order the matrix-core operands want them, so
+// both the writes and the reads are 16 bytes per lane, lane after lane).  One barrier per 128
+// keys.  A token at absolute position p sees keys lo..p only (lo = 0, or p - window + 1),
+// whatever portion it arrived in; a wave skips the 32-key chunks none of its columns sees.
+//
+// The host sorts the tiles by the number of keys they walk and deals them out to the blocks
+// of a kv head in rounds, back and forth, so that every block gets about the same work.
 #include "attention_mfma.h"
+
+#define KEYS_PER_ROUND 128
 
 template <int HD, int CB>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2 : 1))) void attention_tiles_kernel(
     bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q, long q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ q_start, const int* __restrict__ kv_len_of,
-    const int* __restrict__ tile_req, const int* __restrict__ tile_q0, int nh, int nkv, int page_size, float scale,
-    int window, long num_pages, int TQ) {
-  const int lane = threadIdx.x % 64, wave = threadIdx.x / 64;
+    const int* __restrict__ tile_req, const int* __restrict__ tile_q0, const int* __restrict__ order, int rounds, int nh,
+    int nkv, int page_size, float scale, int window, long num_pages_l, int TQ) {
+  constexpr int F = HD / 8;                       // 16-byte operand fragments per lane and 32 keys: keys HD/16, values HD/16
+  extern __shared__ __attribute__((aligned(16))) u32x4_t staged[];   // [2 buffers][4 chunks][F][64 lanes]
+  __shared__ int present[2][4][2];                // is the page of a 16-key tile there
+  const int lane = threadIdx.x % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
   const int lr = lane % 16, lg = lane / 16;
-  const int tile = gridDim.x - 1 - blockIdx.x, g = blockIdx.y;   // later tiles see more keys: start them first
-  const int G = nh / nkv;
-  const int r = tile_req[tile], q0 = tile_q0[tile];
-  const int qs = q_start[r];
-  const int q_len = q_start[r + 1] - qs;
-  const int kv_len = kv_len_of[r];
-  const int* bt = block_table + (long)r * table_width;
+  const int g = blockIdx.y, G = nh / nkv, B = gridDim.x;
+  // blocks of the second half of the kv heads take the deal in reverse: two blocks that end
+  // up on one compute unit then tend to hold a long and a short tile
+  const int seat = (2 * blockIdx.y >= gridDim.y) ? B - 1 - (int)blockIdx.x : (int)blockIdx.x;
+  const int num_pages = (int)(num_pages_l < 0x7fffffffL ? num_pages_l : 0x7fffffffL);
+  const float scale_log2 = scale * PI_LOG2E;
+  KVLaneOffsets<HD> off;
+  off.set(page_size, lane);
+  const int step_blk = KEYS_PER_ROUND / page_size, step_slot = KEYS_PER_ROUND % page_size;
 
-  AttnState<HD, CB> st;
-  attn_init(st);
-  long rows[CB];
-  int heads[CB];
-  bool valid[CB];
-  // over the wave's real columns: the first and last key any of them sees (the walk), and the
-  // keys all of them see (no masking needed there)
-  int lo_min = 0x7fffffff, lo_max = 0, pos_min = 0x7fffffff, pos_max = -1;
+  for (int round = 0; round < rounds; ++round) {
+    const int tile = order[round * B + seat];
+    if (tile < 0) continue;                        // same for the whole block
+    const int r = tile_req[tile], q0 = tile_q0[tile];
+    const int qs = q_start[r];
+    const int q_len = q_start[r + 1] - qs;
+    const int kv_len = kv_len_of[r];
+    const int n_tok = min(TQ, q_len - q0);
+    const int pos0 = kv_len - q_len + q0;          // position of the tile's first token
+    auto first_key = [&](int pos) { return (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0; };
+    // keys the block walks
+    const int sc0 = first_key(pos0) / KEYS_PER_ROUND, sc1 = (pos0 + n_tok - 1) / KEYS_PER_ROUND + 1;
+    // tokens of this wave's columns, and the keys all / any of them see
+    const int tok_a = (wave * CB * 16) / G, tok_b = min(((wave + 1) * CB * 16 - 1) / G, n_tok - 1);
+    const bool active = tok_a < n_tok;
+    const int see_any_lo = first_key(pos0 + tok_a), see_any_hi = pos0 + tok_b;
+    const int see_all_lo = first_key(pos0 + tok_b), see_all_hi = pos0 + tok_a;
+
+    AttnState<HD, CB> st;
+    attn_init(st);
+    long rows[CB];
+    int heads[CB];
+    bool valid[CB];
 #pragma unroll
-  for (int c = 0; c < CB; ++c) {
-    const int col = (wave * CB + c) * 16 + lr;
-    const int tok = col / G;
-    valid[c] = tok < TQ && q0 + tok < q_len;
-    const int pos = kv_len - q_len + q0 + tok;
-    rows[c] = qs + q0 + tok;
-    heads[c] = g * G + col % G;
-    // padding columns are computed on zeros, see everything and are never stored
-    st.pos[c] = valid[c] ? pos : 0x7fffffff;
-    st.lo[c] = (valid[c] && window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
-    attn_load_q(st, c, q, q_stride, rows[c], heads[c], valid[c], lane);
-    if (valid[c]) {
-      lo_min = min(lo_min, st.lo[c]);
-      lo_max = max(lo_max, st.lo[c]);
-      pos_min = min(pos_min, pos);
-      pos_max = max(pos_max, pos);
+    for (int c = 0; c < CB; ++c) {
+      const int col = (wave * CB + c) * 16 + lr;
+      const int tok = col / G;
+      valid[c] = tok < n_tok;
+      rows[c] = qs + q0 + tok;
+      heads[c] = g * G + col % G;
+      // padding columns are computed on zeros, see everything and are never stored
+      st.pos[c] = valid[c] ? pos0 + tok : 0x7fffffff;
+      st.lo[c] = valid[c] ? first_key(pos0 + tok) : 0;
+      attn_load_q(st, c, q, q_stride, rows[c], heads[c], valid[c], lane);
     }
-  }
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    lo_min = min(lo_min, __shfl_xor(lo_min, off, 64));
-    lo_max = max(lo_max, __shfl_xor(lo_max, off, 64));
-    pos_min = min(pos_min, __shfl_xor(pos_min, off, 64));
-    pos_max = max(pos_max, __shfl_xor(pos_max, off, 64));
-  }
-  if (pos_max < 0) return;   // no column of this wave is a real query
 
-  attn_walk<HD, CB>(st, lo_min / 32, pos_max / 32 + 1, (lo_max + 31) / 32, (pos_min + 1) / 32 - 1, k_cache, v_cache, bt,
-                    table_width, kv_len, nkv, g, page_size, num_pages, scale * PI_LOG2E, lane);
-  attn_finish(st);
+    // this wave's 32 keys of every 128: where they lie
+    PageCursor cur;
+    cur.start(block_table + (long)r * table_width, table_width, kv_len, page_size, sc0 * KEYS_PER_ROUND + wave * 32);
+    KVChunk<HD> pre;
+    auto fetch = [&]() {
+      PageCursor two = cur;                        // the chunk's two tiles
+      const ChunkPages cp = two.next();
+      attn_load<HD>(pre, cp, k_cache, v_cache, off, nkv, g, page_size, num_pages);
+      cur.key += KEYS_PER_ROUND;
+      cur.blk += step_blk;
+      cur.slot += step_slot;
+      if (cur.slot >= page_size) { cur.slot -= page_size; ++cur.blk; }
+    };
+    auto stash = [&](int buf) {
+      u32x4_t* mine = staged + ((buf * 4 + wave) * F) * 64 + lane;
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int ks = 0; ks < HD / 32; ++ks) mine[(t * (HD / 32) + ks) * 64] = pre.k[t][ks].n;
+#pragma unroll
+      for (int db = 0; db < HD / 16; ++db)
+        mine[(HD / 16 + db) * 64] = u32x4_t{pre.v[db].d[0].x, pre.v[db].d[0].y, pre.v[db].d[1].x, pre.v[db].d[1].y};
+      if (lane < 2) present[buf][wave][lane] = lane == 0 ? pre.have[0] : pre.have[1];
+    };
+
+    fetch();
+    stash(0);
+    __syncthreads();
+    for (int sc = sc0; sc < sc1; ++sc) {
+      const int buf = (sc - sc0) & 1;
+      fetch();                                     // the next 128 keys (past the end: no pages, page 0 is read)
+      if (active) {
+#pragma unroll 1
+        for (int j = 0; j < 4; ++j) {
+          const int key0 = sc * KEYS_PER_ROUND + j * 32;
+          if (key0 > see_any_hi || key0 + 31 < see_any_lo) continue;
+          KVChunk<HD> kv;
+          const u32x4_t* from = staged + ((buf * 4 + j) * F) * 64 + lane;
+#pragma unroll
+          for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int ks = 0; ks < HD / 32; ++ks) kv.k[t][ks].n = from[(t * (HD / 32) + ks) * 64];
+#pragma unroll
+          for (int db = 0; db < HD / 16; ++db) kv.v[db].n = from[(HD / 16 + db) * 64];
+          kv.have[0] = __builtin_amdgcn_readfirstlane(present[buf][j][0]) != 0;
+          kv.have[1] = __builtin_amdgcn_readfirstlane(present[buf][j][1]) != 0;
+          const bool masked = key0 < see_all_lo || key0 + 31 > see_all_hi || !kv.have[0] || !kv.have[1];
+          attn_compute<HD, CB>(st, kv, key0, scale_log2, masked, lane);
+        }
+      }
+      stash(buf ^ 1);
+      __syncthreads();
+    }
+    attn_finish(st);
 
 #pragma unroll
-  for (int c = 0; c < CB; ++c) {
-    if (!valid[c]) continue;
-    const float inv = 1.0f / st.l[c];
-    bf16_t* o = out + rows[c] * out_stride + (long)heads[c] * HD + lg * 4;
+    for (int c = 0; c < CB; ++c) {
+      if (!valid[c]) continue;
+      const float inv = 1.0f / st.l[c];
+      bf16_t* o = out + rows[c] * out_stride + (long)heads[c] * HD + lg * 4;
 #pragma unroll
-    for (int db = 0; db < HD / 16; ++db) {
-      uint2 w;
-      w.x = pack_bf16x2(st.o[db][c][0] * inv, st.o[db][c][1] * inv);
-      w.y = pack_bf16x2(st.o[db][c][2] * inv, st.o[db][c][3] * inv);
-      *reinterpret_cast<uint2*>(o + db * 16) = w;
+      for (int db = 0; db < HD / 16; ++db) {
+        uint2 w;
+        w.x = pack_bf16x2(st.o[db][c][0] * inv, st.o[db][c][1] * inv);
+        w.y = pack_bf16x2(st.o[db][c][2] * inv, st.o[db][c][3] * inv);
+        *reinterpret_cast<uint2*>(o + db * 16) = w;
+      }
     }
   }
 }
@@ -90,22 +154,37 @@ extern "C" int pi_attention_tile_rows(int nh, int nkv, int hd) {
   return cols / (nh / nkv);
 }
 
+// Shared memory of one block: two buffers of 128 keys and their values.
+static size_t tiles_lds_bytes(int hd) { return (size_t)2 * 4 * (hd / 8) * 64 * 16; }
+
+// `order`: [rounds, seats] tile indices (-1: none), the host's deal of the tiles to `seats`
+// blocks per kv head.
 extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void* q, long q_stride, const void* k_cache,
                                          const void* v_cache, const int* block_table, int table_width, const int* q_start,
-                                         const int* kv_len, const int* tile_req, const int* tile_q0, int num_tiles, int nh,
-                                         int nkv, int hd, int page_size, float scale, int window, long num_pages,
-                                         hipStream_t stream) {
-  PI_REQUIRE(num_tiles > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad sizes tiles=%d heads=%d kv_heads=%d", num_tiles, nh, nkv);
+                                         const int* kv_len, const int* tile_req, const int* tile_q0, const int* order,
+                                         int rounds, int seats, int nh, int nkv, int hd, int page_size, float scale,
+                                         int window, long num_pages, hipStream_t stream) {
+  PI_REQUIRE(rounds > 0 && seats > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad sizes rounds=%d seats=%d heads=%d kv_heads=%d", rounds, seats, nh, nkv);
   PI_REQUIRE(hd == 64 || hd == 128, "attention_prefill: head_dim %d is not 64 or 128", hd);
   PI_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_prefill: page size %d must be a multiple of 16", page_size);
+  PI_REQUIRE(table_width >= 1, "attention_prefill: empty block table");
   const int TQ = pi_attention_tile_rows(nh, nkv, hd);
   PI_REQUIRE(TQ >= 1, "attention_prefill: %d heads per kv head do not fit a block", nh / nkv);
   PI_REQUIRE(nkv <= 65535, "attention_prefill: too many kv heads (%d)", nkv);
   PI_REQUIRE(out_stride % 4 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "attention_prefill: q / out rows must be 16- / 8-byte aligned");
-  const dim3 grid(num_tiles, nkv), block(256);
-#define GO(H, C) hipLaunchKernelGGL((attention_tiles_kernel<H, C>), grid, block, 0, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, \
+  const size_t lds = tiles_lds_bytes(hd);
+  static bool configured[2] = {false, false};
+  if (!configured[hd == 128]) {
+    const void* fn = hd == 64 ? reinterpret_cast<const void*>(attention_tiles_kernel<64, 2>)
+                              : reinterpret_cast<const void*>(attention_tiles_kernel<128, 2>);
+    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+    if (e != hipSuccess) return pi_fail("attention_prefill: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    configured[hd == 128] = true;
+  }
+  const dim3 grid(seats, nkv), block(256);
+#define GO(H, C) hipLaunchKernelGGL((attention_tiles_kernel<H, C>), grid, block, lds, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, \
                                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, \
-                                    kv_len, tile_req, tile_q0, nh, nkv, page_size, scale, window, num_pages, TQ)
+                                    kv_len, tile_req, tile_q0, order, rounds, nh, nkv, page_size, scale, window, num_pages, TQ)
   if (hd == 64) GO(64, 2); else GO(128, 2);
 #undef GO
   return pi_check_launch("attention_prefill_mfma");

@@ -12,9 +12,12 @@
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float f32x4_t __attribute__((ext_vector_type(4)));
 
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
 union Frag {          // 8 bf16 = 16 bytes, seen as the operand type or as raw words
   bf16x8_t v;
   uint4 q;
+  u32x4_t n;          // the same words as a native vector (selects and copies stay in registers)
   uint2 d[2];
   uint16_t h[8];
 };

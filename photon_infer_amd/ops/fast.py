@@ -15,7 +15,7 @@ from __future__ import annotations
 
 import ctypes
 from dataclasses import dataclass
-from typing import Dict, Optional
+from typing import Dict, List, Optional
 
 import numpy as np
 import torch
@@ -185,8 +185,26 @@ def attention_tile_rows(num_heads: int, num_kv_heads: int, head_dim: int) -> int
     return _lib.load("bf16").pi_attention_tile_rows(num_heads, num_kv_heads, head_dim)
 
 
-def _tiles(ctx, tile_rows: int, device):
-    """Work list of the tile kernel: (request, first token) of every tile; cached on the step."""
+ATTENTION_BLOCKS_PER_UNIT = 2   # blocks of the tile kernel that fit one compute unit (LDS, registers)
+
+
+def deal_tiles(walks: List[int], seats: int) -> np.ndarray:
+    """[rounds, seats] tile indices (-1: none): the tiles sorted by the keys they walk, longest
+    first, dealt to ``seats`` blocks back and forth so that the blocks' sums come out close."""
+    by_work = sorted(range(len(walks)), key=lambda i: -walks[i])
+    rounds = -(-len(by_work) // seats)
+    order = np.full((rounds, seats), -1, np.int32)
+    for k in range(rounds):
+        part = by_work[k * seats:(k + 1) * seats]
+        cols = range(len(part)) if k % 2 == 0 else range(seats - 1, seats - 1 - len(part), -1)
+        for c, t in zip(cols, part):
+            order[k, c] = t
+    return order
+
+
+def _tiles(ctx, tile_rows: int, window: int, num_kv_heads: int, device):
+    """Work list of the tile kernel: (request, first token) of every tile and their deal to the
+    blocks; cached on the step (layers with the same window share it)."""
     cache = getattr(ctx, "_attention_tiles", None)
     if cache is None:
         cache = {}
@@ -194,16 +212,25 @@ def _tiles(ctx, tile_rows: int, device):
             ctx._attention_tiles = cache
         except AttributeError:
             pass
-    hit = cache.get(tile_rows)
+    key = (tile_rows, window, num_kv_heads)
+    hit = cache.get(key)
     if hit is None:
-        req, q0 = [], []
-        for r, n in enumerate(ctx.q_lens):
+        req, q0, walks = [], [], []
+        for r, (n, kv) in enumerate(zip(ctx.q_lens, ctx.kv_lens)):
             for start in range(0, n, tile_rows):
                 req.append(r)
                 q0.append(start)
-        host = np.asarray([req, q0], np.int32)
+                first = kv - n + start                         # position of the tile's first token
+                last = first + min(tile_rows, n - start) - 1
+                lo = max(0, first - window + 1) if window > 0 else 0
+                walks.append(last // 128 - lo // 128 + 1)
+        units = torch.cuda.get_device_properties(device).multi_processor_count
+        seats = max(1, min(len(req), ATTENTION_BLOCKS_PER_UNIT * units // max(1, num_kv_heads)))
+        order = deal_tiles(walks, seats)
+        host = np.concatenate([np.asarray(req, np.int32), np.asarray(q0, np.int32), order.reshape(-1)])
         dev = torch.from_numpy(host).to(device)
-        hit = cache[tile_rows] = (dev[0], dev[1], len(req))
+        n = len(req)
+        hit = cache[key] = (dev[:n], dev[n:2 * n], dev[2 * n:], order.shape[0], seats)
     return hit
 
 
@@ -236,11 +263,11 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
     tile_rows = attention_tile_rows(num_heads, num_kv_heads, head_dim)
     if tile_rows < 1:
         return False
-    tile_req, tile_q0, num_tiles = _tiles(ctx, tile_rows, q.device)
+    tile_req, tile_q0, order, rounds, seats = _tiles(ctx, tile_rows, int(window), num_kv_heads, q.device)
     _lib.call("bf16", "pi_attention_prefill_mfma", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
               k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
-              ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(), num_tiles,
-              num_heads, num_kv_heads, head_dim, page_size, float(scale), int(window), pages, _stream())
+              ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(), order.data_ptr(),
+              rounds, seats, num_heads, num_kv_heads, head_dim, page_size, float(scale), int(window), pages, _stream())
     return True
 
 

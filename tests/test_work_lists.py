@@ -1,0 +1,40 @@
+"""Host-side work lists of the kernels (no GPU needed)."""
+import random
+
+import numpy as np
+import pytest
+
+from photon_infer_amd.ops.fast import deal_tiles, decode_splits
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_every_tile_is_dealt_exactly_once(seed):
+    rng = random.Random(seed)
+    walks = [rng.randint(1, 40) for _ in range(rng.randint(1, 300))]
+    seats = rng.randint(1, 70)
+    order = deal_tiles(walks, seats)
+    assert order.shape[1] == seats and order.dtype == np.int32
+    dealt = sorted(int(t) for t in order.reshape(-1) if t >= 0)
+    assert dealt == list(range(len(walks)))
+
+
+def test_the_deal_evens_out_the_work():
+    # a causal prompt: tile i walks i + 1 key ranges
+    walks = list(range(1, 129))
+    order = deal_tiles(walks, 32)
+    sums = [sum(walks[t] for t in order[:, seat] if t >= 0) for seat in range(32)]
+    assert max(sums) - min(sums) <= 1
+    # the first round holds the longest tiles
+    assert sorted(walks[t] for t in order[0]) == list(range(97, 129))
+
+
+def test_fewer_tiles_than_seats():
+    order = deal_tiles([3, 9], 8)
+    assert order.shape == (1, 8)
+    assert list(order[0][:2]) == [1, 0] and all(t == -1 for t in order[0][2:])
+
+
+def test_decode_splits_fill_the_chip_but_respect_short_contexts():
+    assert decode_splits(64, 8) < decode_splits(8, 8) <= 32
+    assert decode_splits(1, 8, max_kv_len=100) == 1
+    assert decode_splits(1, 8, max_kv_len=4096) > 1
