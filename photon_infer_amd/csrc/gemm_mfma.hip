@@ -1,12 +1,13 @@
 // bfloat16 matrix product on the matrix cores for many rows (prompts):
 //   C[M, N] (+)= A[M, K] . W[N, K]^T, float32 accumulation.
-// Block tile 128 x 128, reduction slab 64, four waves in 2 x 2, each wave 64 x 64 as 4 x 4
-// tiles of v_mfma_f32_16x16x32_bf16.  Slabs go global -> registers -> LDS (double buffered,
+// Block tile 128 x 128, reduction slab 64, four waves in 2 x 2, each wave 64 x 64 as 2 x 2
+// tiles of v_mfma_f32_32x32x16_bf16.  Slabs go global -> registers -> LDS (double buffered,
 // rows padded to 144 bytes so 16-byte fragment reads do not collide on banks).
 //
 // Epilogues: store bfloat16, store float32, add into float32 (the residual stream), or
-// SwiGLU: with gate and up rows interleaved in blocks of 16 in W, a lane holds the gate and
-// the up value of the same (row, feature) and stores silu(gate) * up directly.
+// SwiGLU: with gate and up rows interleaved in blocks of 16 in W, the gate and the up value of
+// the same (row, feature) sit 16 lanes apart; one row swap brings them together and
+// silu(gate) * up is stored directly.
 //
 // Any M and N (edges are zero-filled on load and skipped on store); K must be a multiple of
 // 8 and row strides multiples of 8 so that 16-byte loads stay aligned.  Each output row
@@ -23,7 +24,11 @@ PI_DEFINE_MODULE(bf16)
 
 enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACCUM = 2, EPI_SWIGLU = 3 };
 
-__device__ inline float silu_mul(float g, float u) { return g / (1.0f + expf(-g)) * u; }
+// silu(g) * u for a bfloat16 result: the hardware exponential and reciprocal (1 ulp each) are
+// far inside the rounding of the store
+__device__ inline float silu_mul(float g, float u) {
+  return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g)) * u;
+}
 
 template <int EPI>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ A, long lda,
@@ -78,66 +83,269 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
     }
   };
 
-  f32x4_t acc[4][4];
+  f32x16_t acc[2][2];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   const int slabs = (k_hi - k_lo + BK - 1) / BK;
   load_slab(k_lo);
   store_slab(0);
   __syncthreads();
-  const int frow = lane % 16, fk = (lane / 16) * 8;
+  // 32 x 32 x 16 instruction: a lane reads row lane % 32, 16 bytes at k = (lane / 32) * 8; with
+  // rows 144 bytes apart the 16 lanes served together fall on distinct banks
+  const int frow = lane % 32, fk = (lane / 32) * 8;
   for (int s = 0; s < slabs; ++s) {
     const int buf = s & 1;
     if (s + 1 < slabs) load_slab(k_lo + (s + 1) * BK);
     const uint16_t* a_base = As + buf * TILE_ELEMS + (wm * 64 + frow) * LDS_ROW + fk;
     const uint16_t* w_base = Ws + buf * TILE_ELEMS + (wn * 64 + frow) * LDS_ROW + fk;
 #pragma unroll
-    for (int ks = 0; ks < BK / 32; ++ks) {
-      Frag a[4], b[4];
+    for (int ks = 0; ks < BK / 16; ++ks) {
+      Frag a[2], b[2];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) a[i].q = *reinterpret_cast<const uint4*>(a_base + i * 16 * LDS_ROW + ks * 32);
+      for (int i = 0; i < 2; ++i) a[i].n = *reinterpret_cast<const u32x4_t*>(a_base + i * 32 * LDS_ROW + ks * 16);
 #pragma unroll
-      for (int j = 0; j < 4; ++j) b[j].q = *reinterpret_cast<const uint4*>(w_base + j * 16 * LDS_ROW + ks * 32);
+      for (int j = 0; j < 2; ++j) b[j].n = *reinterpret_cast<const u32x4_t*>(w_base + j * 32 * LDS_ROW + ks * 16);
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < 2; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = mfma16(a[i], b[j], acc[i][j]);
+        for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
     }
     if (s + 1 < slabs) store_slab(buf ^ 1);
     __syncthreads();
   }
 
-  // epilogue: acc[i][j][r] is C[m0 + wm*64 + i*16 + (lane/16)*4 + r][n0 + wn*64 + j*16 + lane%16]
-  const int crow = (lane / 16) * 4, ccol = lane % 16;
+  // acc[i][j][v] is C[m0 + wm*64 + i*32 + 8*(v/4) + 4*(lane/32) + v%4][n0 + wn*64 + j*32 + lane%32]
+  const int half = lane / 32, ccol = lane % 32;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
+  for (int i = 0; i < 2; ++i)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const long m = m0 + wm * 64 + i * 16 + crow + r;
-      if (m >= M) continue;
-      if (EPI == EPI_SWIGLU) {
-        bf16_t* C = reinterpret_cast<bf16_t*>(Cv);
+    for (int j = 0; j < 2; ++j) {
+      const long nb = n0 + wn * 64 + j * 32;
 #pragma unroll
-        for (int j = 0; j < 4; j += 2) {
-          const long n = n0 + wn * 64 + j * 16 + ccol;        // gate column; up is at n + 16
-          if (n + 16 < N) C[m * ldc + (n0 + wn * 64 + j * 16) / 2 + ccol] = from_float<bf16_t>(silu_mul(acc[i][j][r], acc[i][j + 1][r]));
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const long n = n0 + wn * 64 + j * 16 + ccol;
-          if (n >= N) continue;
-          if (EPI == EPI_BF16) reinterpret_cast<bf16_t*>(Cv)[m * ldc + n] = from_float<bf16_t>(acc[i][j][r]);
-          if (EPI == EPI_F32) reinterpret_cast<float*>(Cv)[m * ldc + n] = acc[i][j][r];
-          if (EPI == EPI_ACCUM) reinterpret_cast<float*>(Cv)[m * ldc + n] += acc[i][j][r];
+      for (int v = 0; v < 16; ++v) {
+        const long m = m0 + wm * 64 + i * 32 + 8 * (v / 4) + 4 * half + v % 4;
+        if (EPI == EPI_SWIGLU) {
+          // columns 0..15 of a tile are gate rows of W, 16..31 the up rows of the same features:
+          // the swap leaves the gate value in both 16-lane rows of one result and the up value
+          // in both rows of the other; the lower rows store
+#if defined(__HIP_DEVICE_COMPILE__)
+          const unsigned bits = __float_as_uint(acc[i][j][v]);
+          auto gu = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+          if (ccol < 16 && m < M && nb + ccol + 16 < N)
+            reinterpret_cast<bf16_t*>(Cv)[m * ldc + nb / 2 + ccol] = from_float<bf16_t>(silu_mul(__uint_as_float(gu[0]), __uint_as_float(gu[1])));
+#endif
+        } else {
+          const long n = nb + ccol;
+          if (m >= M || n >= N) continue;
+          if (EPI == EPI_BF16) reinterpret_cast<bf16_t*>(Cv)[m * ldc + n] = from_float<bf16_t>(acc[i][j][v]);
+          if (EPI == EPI_F32) reinterpret_cast<float*>(Cv)[m * ldc + n] = acc[i][j][v];
+          if (EPI == EPI_ACCUM) reinterpret_cast<float*>(Cv)[m * ldc + n] += acc[i][j][v];
         }
       }
     }
+}
+
+// ---------------------------------------------------------------------------------------------
+// The same product with block tile 256 x 256 for problems that have enough of them to fill the
+// chip and a k that is a multiple of the slab: four waves in 2 x 2, each 128 x 128 as 4 x 4
+// tiles of v_mfma_f32_32x32x16_bf16.  Per 16 k a wave reads 8 fragments from LDS for 16
+// matrix-core instructions, half the LDS traffic per flop of the 128 x 128 kernel.  The
+// accumulators alone are 256 registers, so there is one wave per SIMD and nothing else to fill
+// its idle cycles: every load, LDS access and address computation has to be issued in the
+// shadow of a matrix-core instruction (32 cycles each).  Hence no branch in the loop (rows
+// beyond the matrix are clamped on load and skipped on store), global loads through a buffer
+// descriptor (a scalar base that moves with k plus fixed 32-bit lane offsets, no vector
+// arithmetic per slab), and scheduling hints that deal the memory instructions out between
+// the matrix-core ones.  A slab's global loads are issued a whole slab before they are stored.
+// Per output element the sum over k runs in ascending k, as in the small kernel.
+#define GM 256
+#define GN 256
+#define BIG_TILE_ELEMS (GM * LDS_ROW)
+#define PI_SCHED_MFMA 0x008
+#define PI_SCHED_VMEM_READ 0x020
+#define PI_SCHED_DS_READ 0x100
+#define PI_SCHED_DS_WRITE 0x200
+
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_mfma_big_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ A, long lda,
+                                                            const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
+                                                            int tiles_n, int k_per_split) {
+  extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
+  uint16_t* As = lds;                           // [2][GM][LDS_ROW]
+  uint16_t* Ws = lds + 2 * BIG_TILE_ELEMS;      // [2][GN][LDS_ROW]
+  const int tid = threadIdx.x, lane = tid % 64;
+  const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
+  const int wm = wave / 2, wn = wave % 2;
+  const int k_lo = blockIdx.y * k_per_split;
+  const int k_hi = min(K, k_lo + k_per_split);
+  if (gridDim.y > 1) Cv = reinterpret_cast<float*>(Cv) + (long)blockIdx.y * M * ldc;
+  const int tiles_m = gridDim.x / tiles_n;
+  int tile_m, tile_n;
+  if (tiles_n % 8 == 0) {                       // a die streams its own slice of W, see above
+    const int die = blockIdx.x % 8, local = blockIdx.x / 8;
+    tile_n = die * (tiles_n / 8) + local / tiles_m;
+    tile_m = local % tiles_m;
+  } else {
+    tile_m = blockIdx.x / tiles_n;
+    tile_n = blockIdx.x % tiles_n;
+  }
+  const long m0 = (long)tile_m * GM, n0 = (long)tile_n * GN;
+
+  // global -> registers: thread t moves 16-byte chunk t % 8 of rows lrow + 32 p of both operands
+  const int lgrp = tid / 8, lchunk = tid % 8;
+  const int lrow = (lgrp / 16) * 16 + ((lgrp / 8) % 2) * 4 + (lgrp % 8) / 2 + 8 * (lgrp % 2);
+  const int a_rows = (int)min((long)GM, M - m0), w_rows = (int)min((long)GN, N - n0);
+#if defined(__HIP_DEVICE_COMPILE__)
+  // descriptors: base of the block's rows at k_lo, length up to the end of its last row; built
+  // from values made scalar by hand so that the loads take them from scalar registers
+  auto descriptor = [](const bf16_t* base, long bytes) {
+    const uint64_t v = reinterpret_cast<uint64_t>(base);
+    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+    void* p = reinterpret_cast<void*>((static_cast<uint64_t>(hi) << 32) | lo);
+    return __builtin_amdgcn_make_buffer_rsrc(p, 0, __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000);
+  };
+  const __amdgpu_buffer_rsrc_t a_src = descriptor(A + m0 * lda + k_lo, ((long)(a_rows - 1) * lda + (k_hi - k_lo)) * 2);
+  const __amdgpu_buffer_rsrc_t w_src = descriptor(W + n0 * ldw + k_lo, ((long)(w_rows - 1) * ldw + (k_hi - k_lo)) * 2);
+#endif
+  unsigned a_off[8], w_off[8];
+#pragma unroll
+  for (int p = 0; p < 8; ++p) {
+    a_off[p] = (unsigned)(min(lrow + 32 * p, a_rows - 1) * (int)lda + lchunk * 8) * 2u;
+    w_off[p] = (unsigned)(min(lrow + 32 * p, w_rows - 1) * (int)ldw + lchunk * 8) * 2u;
+  }
+  u32x4_t ra[8], rw[8];
+  const int slabs = (k_hi - k_lo) / BK;
+  auto load_slab = [&](int s) {
+    const int kbytes = min(s, slabs - 1) * BK * 2;     // past the last slab: read it again, unused
+#if defined(__HIP_DEVICE_COMPILE__)
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      ra[p] = __builtin_amdgcn_raw_buffer_load_b128(a_src, a_off[p], kbytes, 0);
+      rw[p] = __builtin_amdgcn_raw_buffer_load_b128(w_src, w_off[p], kbytes, 0);
+    }
+#endif
+  };
+  auto store_slab = [&](int buf) {
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      const int off = (lrow + 32 * p) * LDS_ROW + lchunk * 8;
+      *reinterpret_cast<u32x4_t*>(As + buf * BIG_TILE_ELEMS + off) = ra[p];
+      *reinterpret_cast<u32x4_t*>(Ws + buf * BIG_TILE_ELEMS + off) = rw[p];
+    }
+  };
+
+  f32x16_t acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+
+  const int frow = lane % 32, fk = (lane / 32) * 8;
+  Frag fa[2][4], fb[2][4];
+  auto read_frags = [&](int which, int buf, int ks) {   // ks: which 16 k of the slab
+    const uint16_t* a_base = As + buf * BIG_TILE_ELEMS + (wm * 128 + frow) * LDS_ROW + fk + ks * 16;
+    const uint16_t* w_base = Ws + buf * BIG_TILE_ELEMS + (wn * 128 + frow) * LDS_ROW + fk + ks * 16;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) fa[which][i].n = *reinterpret_cast<const u32x4_t*>(a_base + i * 32 * LDS_ROW);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) fb[which][j].n = *reinterpret_cast<const u32x4_t*>(w_base + j * 32 * LDS_ROW);
+  };
+  auto products = [&](int which) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[i][j] = mfma32(fa[which][i], fb[which][j], acc[i][j]);
+  };
+  // the order wanted inside one scheduling region: one matrix-core instruction, then one of
+  // each kind of memory instruction named, `n` times; the rest of the 16 after that
+#define PI_DEAL(n, kind_a, kind_b)                                                   \
+  _Pragma("unroll") for (int d_ = 0; d_ < n; ++d_) {                                 \
+    __builtin_amdgcn_sched_group_barrier(PI_SCHED_MFMA, 1, 0);                       \
+    if (kind_a) __builtin_amdgcn_sched_group_barrier(kind_a, 1, 0);                  \
+    if (kind_b) __builtin_amdgcn_sched_group_barrier(kind_b, 1, 0);                  \
+  }
+
+  load_slab(0);
+  store_slab(0);
+  __syncthreads();
+  load_slab(1);
+  read_frags(0, 0, 0);
+  for (int s = 0; s < slabs; ++s) {
+    const int buf = s & 1;
+    read_frags(1, buf, 1);
+    products(0);
+    PI_DEAL(8, PI_SCHED_DS_READ, 0)
+    PI_DEAL(8, 0, 0)
+    read_frags(0, buf, 2);
+    products(1);
+    PI_DEAL(8, PI_SCHED_DS_READ, 0)
+    PI_DEAL(8, 0, 0)
+    read_frags(1, buf, 3);
+    products(0);
+    store_slab(buf ^ 1);            // slab s + 1, loaded during the previous slab's last step
+    PI_DEAL(8, PI_SCHED_DS_READ, PI_SCHED_DS_WRITE)
+    PI_DEAL(8, PI_SCHED_DS_WRITE, 0)
+    __syncthreads();
+    load_slab(s + 2);
+    read_frags(0, buf ^ 1, 0);
+    products(1);
+    PI_DEAL(8, PI_SCHED_VMEM_READ, PI_SCHED_DS_READ)
+    PI_DEAL(8, PI_SCHED_VMEM_READ, 0)
+  }
+#undef PI_DEAL
+
+  // acc[i][j][v] is C[m0 + wm*128 + i*32 + 8*(v/4) + 4*(lane/32) + v%4][n0 + wn*128 + j*32 + lane%32].
+  // Offsets inside the wave's 128 x 128 corner are 32-bit (the host checks 128 * ldc fits).
+  const int half = lane / 32, ccol = lane % 32;
+  const long mw = m0 + wm * 128, nw = n0 + wn * 128;
+  const int rows_left = (int)min((long)128, M - mw), cols_left = (int)min((long)128, N - nw);   // may be <= 0
+  const int ld = (int)ldc;
+  if (EPI == EPI_SWIGLU) {
+    // columns 0..15 of a tile are gate rows of W, 16..31 the up rows of the same features: bring
+    // the two together (the swap leaves the gate value in both 16-lane rows of one result and
+    // the up value in both rows of the other); the lower rows store
+    bf16_t* C = reinterpret_cast<bf16_t*>(Cv) + mw * ldc + nw / 2;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+          const unsigned bits = __float_as_uint(acc[i][j][v]);
+          auto gu = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
+          const int rl = i * 32 + 8 * (v / 4) + 4 * half + v % 4;
+          if (ccol < 16 && rl < rows_left && j * 32 + ccol + 16 < cols_left)
+            C[rl * ld + j * 16 + ccol] = from_float<bf16_t>(silu_mul(__uint_as_float(gu[0]), __uint_as_float(gu[1])));
+#endif
+        }
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+          const int rl = i * 32 + 8 * (v / 4) + 4 * half + v % 4, cl = j * 32 + ccol;
+          if (rl >= rows_left || cl >= cols_left) continue;
+          const int off = rl * ld + cl;
+          if (EPI == EPI_BF16) (reinterpret_cast<bf16_t*>(Cv) + mw * ldc + nw)[off] = from_float<bf16_t>(acc[i][j][v]);
+          if (EPI == EPI_F32) (reinterpret_cast<float*>(Cv) + mw * ldc + nw)[off] = acc[i][j][v];
+          if (EPI == EPI_ACCUM) (reinterpret_cast<float*>(Cv) + mw * ldc + nw)[off] += acc[i][j][v];
+        }
   }
 }
+
+static const size_t kBigLdsBytes = 4 * BIG_TILE_ELEMS * sizeof(uint16_t);   // 147,456 bytes
+#define BIG_MIN_TILES 192      // enough 256 x 256 tiles (times k pieces) to occupy most of the chip
 
 static const size_t kLdsBytes = 4 * TILE_ELEMS * sizeof(uint16_t);   // 73,728 bytes
 
@@ -151,10 +359,24 @@ static int launch(void* C, long ldc, const void* A, long lda, const void* W, lon
     if (e != hipSuccess) return pi_fail("gemm_mfma: cannot reserve %zu bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
     configured = true;
   }
-  const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
   int kps = ceil_div(K, splits);
   kps = ((kps + BK - 1) / BK) * BK;
   splits = ceil_div(K, kps);
+  const long big_tiles = (long)ceil_div(M, GM) * ceil_div(N, GN);
+  if (big_tiles * splits >= BIG_MIN_TILES && big_tiles < 2147483647L && ldc < (1L << 23) && K % BK == 0 &&
+      256 * lda < (1L << 30) && 256 * ldw < (1L << 30)) {
+    static bool big_configured = false;
+    if (!big_configured) {
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma_big_kernel<EPI>),
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kBigLdsBytes);
+      if (e != hipSuccess) return pi_fail("gemm_mfma: cannot reserve %zu bytes of LDS: %s", kBigLdsBytes, hipGetErrorString(e));
+      big_configured = true;
+    }
+    hipLaunchKernelGGL((gemm_mfma_big_kernel<EPI>), dim3((unsigned)big_tiles, splits), dim3(256), kBigLdsBytes, stream, C, ldc,
+                       (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, ceil_div(N, GN), kps);
+    return pi_check_launch("gemm_mfma_big");
+  }
+  const int tiles_m = ceil_div(M, BM), tiles_n = ceil_div(N, BN);
   hipLaunchKernelGGL((gemm_mfma_kernel<EPI>), dim3((unsigned)tiles_m * tiles_n, splits), dim3(256), kLdsBytes, stream, C, ldc,
                      (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, tiles_n, kps);
   return pi_check_launch("gemm_mfma");

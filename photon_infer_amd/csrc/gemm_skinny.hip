@@ -41,8 +41,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
   const int kb0 = blockIdx.y * k_per_block;
   const int kb1 = min(K, kb0 + k_per_block);
   const int per_wave = ((kb1 - kb0 + 4 * KSTEP - 1) / (4 * KSTEP)) * KSTEP;
-  const int k0 = __builtin_amdgcn_readfirstlane(kb0 + wave * per_wave);   // the same in the whole wave
-  const int k1 = __builtin_amdgcn_readfirstlane(min(kb1, k0 + per_wave));
+  const int k0 = kb0 + wave * per_wave;
+  const int k1 = min(kb1, k0 + per_wave);
 
   // rows beyond N / tokens beyond M read the last valid row; their results are never stored
   const bf16_t* wrow[2];
@@ -58,48 +58,27 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
 #pragma unroll
     for (int c = 0; c < MB; ++c) acc[t][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  // Whole steps, two in flight: the loads of the next step are issued before the products of
-  // the current one, and the loop body has no branch, so the compiler can wait by count.
-  // A load past the last whole step re-reads that step and is not used.
-  const int nfull = k1 > k0 ? (k1 - k0) / KSTEP : 0;
-  if (nfull > 0) {
-    const int klast = k0 + (nfull - 1) * KSTEP;
-    Frag wa[2][2], xa[MB][2], wb[2][2], xb[MB][2];
-    auto load = [&](Frag (&w)[2][2], Frag (&x)[MB][2], int kk) {
-      kk = min(kk, klast);
+  int kk = k0;
+  for (; kk + KSTEP <= k1; kk += KSTEP) {
+    Frag w[2][2], x[MB][2];
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        w[t][0] = load_frag(wrow[t] + kk);
-        w[t][1] = load_frag(wrow[t] + kk + 8);
-      }
+    for (int t = 0; t < 2; ++t) {
+      w[t][0] = load_frag(wrow[t] + kk);
+      w[t][1] = load_frag(wrow[t] + kk + 8);
+    }
+#pragma unroll
+    for (int c = 0; c < MB; ++c) {
+      x[c][0] = load_frag(xrow[c] + kk);
+      x[c][1] = load_frag(xrow[c] + kk + 8);
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
       for (int c = 0; c < MB; ++c) {
-        x[c][0] = load_frag(xrow[c] + kk);
-        x[c][1] = load_frag(xrow[c] + kk + 8);
+        acc[t][c] = mfma16(w[t][0], x[c][0], acc[t][c]);
+        acc[t][c] = mfma16(w[t][1], x[c][1], acc[t][c]);
       }
-    };
-    auto products = [&](const Frag (&w)[2][2], const Frag (&x)[MB][2]) {
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int c = 0; c < MB; ++c) {
-          acc[t][c] = mfma16(w[t][0], x[c][0], acc[t][c]);
-          acc[t][c] = mfma16(w[t][1], x[c][1], acc[t][c]);
-        }
-    };
-    load(wa, xa, k0);
-    int ka = k0;
-    for (int pair = 0; pair < nfull / 2; ++pair, ka += 2 * KSTEP) {
-      load(wb, xb, ka + KSTEP);
-      __builtin_amdgcn_sched_barrier(0);     // keep the loads ahead of the products they overlap
-      products(wa, xa);
-      load(wa, xa, ka + 2 * KSTEP);
-      __builtin_amdgcn_sched_barrier(0);
-      products(wb, xb);
-    }
-    if (nfull % 2) products(wa, xa);   // an odd last step is already loaded
   }
-  const int kk = k0 + nfull * KSTEP;
   if (kk < k1) {  // a last, partial step: 8-element chunks beyond k1 count as zero
     const int ka = kk + lg * 16;
 #pragma unroll

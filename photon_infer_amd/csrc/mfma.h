@@ -26,6 +26,14 @@ __device__ inline f32x4_t mfma16(const Frag& a, const Frag& b, f32x4_t c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, c, 0, 0, 0);
 }
 
+typedef float f32x16_t __attribute__((ext_vector_type(16)));
+
+// 32 x 32 x 16: lane l holds row (column) l % 32 of the operand, k = (l / 32) * 8 .. + 8; of the
+// result it holds column l % 32 and the 16 rows 8 * (v / 4) + 4 * (l / 32) + v % 4, v = 0..15.
+__device__ inline f32x16_t mfma32(const Frag& a, const Frag& b, f32x16_t c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b.v, c, 0, 0, 0);
+}
+
 __device__ inline Frag zero_frag() {
   Frag f;
   f.q = make_uint4(0u, 0u, 0u, 0u);

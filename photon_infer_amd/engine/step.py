@@ -13,7 +13,7 @@ steps left.  Portions of prompts and single decoded tokens mix freely.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Dict, Hashable, List, Optional, Sequence
+from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
@@ -61,7 +61,7 @@ class ModelRunner:
         self.model.load(tensors, self.dtype, self.device)
         del tensors
         self._build_cache()
-        self._graphs: Dict[int, "_DecodeGraph"] = {}
+        self._graphs: Dict[Tuple[int, int], "_DecodeGraph"] = {}
 
     # ------------------------------------------------------------------ cache set-up
     def _build_cache(self) -> None:
@@ -204,9 +204,11 @@ class ModelRunner:
         if any(len(e.tokens) != 1 for e in entries):
             raise RequestError("decode_step takes exactly one token per request")
         self._reserve(entries)
-        graph = self._graphs.get(len(entries))
+        # one graph per batch size and length bucket: the attention kernel's key ranges follow the bucket
+        bucket = ops.decode_length_bucket(max(self.cache.length(e.rid) for e in entries) + 1)
+        graph = self._graphs.get((len(entries), bucket))
         if graph is None:
-            graph = self._graphs[len(entries)] = _DecodeGraph(self, len(entries))
+            graph = self._graphs[(len(entries), bucket)] = _DecodeGraph(self, len(entries), bucket)
         out = graph.run(entries, temperatures, uniforms)
         for e in entries:
             self.cache.commit(e.rid, 1)
@@ -228,15 +230,15 @@ def _upload(parts: Dict[str, np.ndarray], device) -> Dict[str, torch.Tensor]:
 
 
 class _DecodeGraph:
-    """The decode step of one batch size as a HIP graph.
+    """The decode step of one batch size and context-length bucket as a HIP graph.
 
     All metadata lives in one device buffer at fixed addresses (tokens, positions, lengths,
     slots, sampling parameters, block-table rows of full width); a step copies the new values
     in and replays.  Nothing in the graph depends on a host-side number: the attention grid is
-    fixed by the batch size, key ranges are derived on the device from the lengths.
+    fixed by the batch size and the bucket, key ranges are derived on the device from the lengths.
     """
 
-    def __init__(self, runner: "ModelRunner", R: int):
+    def __init__(self, runner: "ModelRunner", R: int, length_bucket: int):
         self.runner, self.R = runner, R
         cache = runner.cache
         self.width = cache.max_blocks
@@ -263,8 +265,7 @@ class _DecodeGraph:
             T=R, R=R, dtype=runner.dtype, token_ids=d["token_ids"], positions=d["positions"],
             req_of_token=d["req_of_token"], q_start=d["q_start"], kv_len=d["kv_len"], slots=d["slots"],
             block_tables={g: d[f"table{g}"].view(R, self.width) for g in range(G)}, logit_rows=d["logit_rows"],
-            q_lens=[1] * R, kv_lens=(), max_q_len=1, max_kv_len=None, all_decode=True)
-        self.ctx.decode_splits_fixed = True       # key ranges by batch size only, not by the lengths of the day
+            q_lens=[1] * R, kv_lens=(), max_q_len=1, max_kv_len=length_bucket, all_decode=True)
         self.temps = d["temps"].view(torch.float32)
         self.uniforms = d["uniforms"].view(torch.float32)
         self.sampled = torch.zeros(R, dtype=torch.int32, device=runner.device)

@@ -379,6 +379,12 @@ _SAMPLE_WS: dict = {}
 
 
 # ----------------------------------------------------------------------------- work lists
+def decode_length_bucket(max_kv_len: int) -> int:
+    """The context-length bucket that decides a decode step's attention key ranges."""
+    from . import fast
+    return fast.decode_length_bucket(max_kv_len)
+
+
 def plan_attention(q_lens, kv_lens, dtype) -> dict:
     """Host-side work lists (int32 arrays to upload with the step's metadata) that the
     matrix-core attention kernels want; empty for the general kernels."""

@@ -234,13 +234,21 @@ def _tiles(ctx, tile_rows: int, window: int, num_kv_heads: int, device):
     return hit
 
 
-def decode_splits(R: int, num_kv_heads: int, max_kv_len: Optional[int] = None) -> int:
+def decode_length_bucket(max_kv_len: int) -> int:
+    """The power of two (at least one key range's worth) that a decode step's longest context
+    is rounded up to.  Key ranges are chosen per bucket, so a step gives the same numbers
+    whether it runs eagerly or replays the graph captured for its bucket."""
+    bucket = DECODE_MIN_KEYS_PER_SPLIT
+    while bucket < max_kv_len:
+        bucket *= 2
+    return bucket
+
+
+def decode_splits(R: int, num_kv_heads: int, max_kv_len: int) -> int:
     """Key ranges per (request, kv head): enough waves to fill the chip, no more than the
-    keys are worth."""
+    keys of the step's length bucket are worth."""
     splits = max(1, min(MAX_DECODE_SPLITS, -(-DECODE_WAVES_WANTED // (R * num_kv_heads))))
-    if max_kv_len is not None:
-        splits = min(splits, max(1, -(-max_kv_len // DECODE_MIN_KEYS_PER_SPLIT)))
-    return splits
+    return min(splits, max(1, decode_length_bucket(max_kv_len) // DECODE_MIN_KEYS_PER_SPLIT))
 
 
 def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
@@ -250,8 +258,7 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
     G = num_heads // num_kv_heads
     R = ctx.R
     if ctx.all_decode and G <= 16:
-        fixed = getattr(ctx, "decode_splits_fixed", False)
-        splits = decode_splits(R, num_kv_heads, None if fixed else ctx.max_kv_len)
+        splits = decode_splits(R, num_kv_heads, ctx.max_kv_len)
         ws = workspace(q.device)
         while splits > 1 and R * num_heads * splits * (head_dim + 4) > ws.attn_part.numel():
             splits -= 1

@@ -130,6 +130,52 @@ def test_gemm_with_swiglu_in_the_epilogue(_ops, M, I, K):
     close(out, want, 2 ** -7, "swiglu on halves")
 
 
+@pytest.mark.parametrize("M,N,K", [(1024, 12288, 192), (1000, 12300, 256), (1000, 12300, 264), (2048, 6200, 72)])
+def test_gemm_on_large_tiles(_ops, M, N, K):
+    """Enough 256 x 256 tiles to fill the chip: the one-wave-per-SIMD kernel, with ragged edges
+    in every dimension and a k that is no multiple of its slab."""
+    _ops.use_fast_kernels(True)
+    a = torch.randn(M, K, generator=gen(M)).to(BF16)
+    w = torch.randn(N, K, generator=gen(N)).to(BF16)
+    want = a.double() @ w.double().t()
+    for c_dtype, rel in ((BF16, 2 ** -8), (F32, 2e-6)):
+        out = torch.empty(M, N, dtype=c_dtype, device=DEV)
+        _ops.gemm(out, a.to(DEV), w.to(DEV))
+        close(out, want, rel, f"large gemm {M}x{N}x{K} {c_dtype}")
+    base = torch.randn(M, N, generator=gen(9))
+    acc = base.clone().to(DEV)
+    _ops.gemm(acc, a.to(DEV), w.to(DEV), accumulate=True)
+    close(acc, want + base.double(), 2e-6, "large gemm accumulate")
+
+
+def test_gemm_on_large_tiles_split_over_k(_ops):
+    """Few output tiles and a long k: pieces over k from the large-tile kernel, summed by materialize."""
+    _ops.use_fast_kernels(True)
+    M, N, K = 2048, 2040, 4104
+    a = (torch.randn(M, K, generator=gen(1)) * 0.25).to(BF16)
+    w = (torch.randn(N, K, generator=gen(2)) * 0.25).to(BF16)
+    base = torch.randn(M, N, generator=gen(3))
+    want = a.double() @ w.double().t() + base.double()
+    x = base.clone().to(DEV)
+    _ops.reset_deferred()
+    _ops.gemm(x, a.to(DEV), w.to(DEV), accumulate=True, may_defer=True)
+    _ops.materialize(x)
+    close(x, want, 2e-6, "k-split large gemm")
+
+
+@pytest.mark.parametrize("M,I,K", [(1000, 6160, 200), (1000, 6160, 192), (2048, 8192, 64)])
+def test_gemm_with_swiglu_on_large_tiles(_ops, M, I, K):
+    _ops.use_fast_kernels(True)
+    a = torch.randn(M, K, generator=gen(M)).to(BF16)
+    g = (torch.randn(I, K, generator=gen(I)) * 0.3).to(BF16)
+    u = (torch.randn(I, K, generator=gen(K)) * 0.3).to(BF16)
+    w_il = torch.stack([g.view(I // 16, 16, K), u.view(I // 16, 16, K)], dim=1).reshape(2 * I, K).contiguous()
+    want = P.swiglu(a.double() @ g.double().t(), a.double() @ u.double().t())
+    out = torch.empty(M, I, dtype=BF16, device=DEV)
+    _ops.gemm_swiglu(out, a.to(DEV), w_il.to(DEV), 16)
+    close(out, want, 2 ** -7, "fused swiglu on large tiles")
+
+
 def test_gemm_reference_vectors(_ops):
     # tests/ops/test_matmul.cpp:90-204
     W = torch.tensor([[1.0, 2.0, 3.0], [4.0, 5.0, 6.0]], device=DEV)

@@ -4,7 +4,7 @@ import random
 import numpy as np
 import pytest
 
-from photon_infer_amd.ops.fast import deal_tiles, decode_splits
+from photon_infer_amd.ops.fast import deal_tiles, decode_length_bucket, decode_splits
 
 
 @pytest.mark.parametrize("seed", range(5))
@@ -35,6 +35,9 @@ def test_fewer_tiles_than_seats():
 
 
 def test_decode_splits_fill_the_chip_but_respect_short_contexts():
-    assert decode_splits(64, 8) < decode_splits(8, 8) <= 32
+    assert decode_splits(64, 8, 4096) < decode_splits(8, 8, 4096) <= 32
     assert decode_splits(1, 8, max_kv_len=100) == 1
     assert decode_splits(1, 8, max_kv_len=4096) > 1
+    # the same key ranges anywhere inside a length bucket: eager steps and graph replays agree
+    assert decode_length_bucket(129) == decode_length_bucket(256) == 256
+    assert decode_splits(4, 8, 1025) == decode_splits(4, 8, 2048)
