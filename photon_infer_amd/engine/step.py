@@ -13,6 +13,7 @@ steps left.  Portions of prompts and single decoded tokens mix freely.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+import gc
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -298,8 +299,16 @@ class _DecodeGraph:
             self._body()
             torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph):
-                self._body()
+            # no garbage collection while the stream is capturing: a collected tensor of some
+            # earlier engine (pinned memory, events) would make calls that a capture forbids
+            collecting = gc.isenabled()
+            gc.disable()
+            try:
+                with torch.cuda.graph(graph):
+                    self._body()
+            finally:
+                if collecting:
+                    gc.enable()
             self.graph = graph
         else:
             self.graph.replay()
