@@ -234,7 +234,7 @@ class _DecodeGraph:
     """The decode step of one batch size and context-length bucket as a HIP graph.
 
     All metadata lives in one device buffer at fixed addresses (tokens, positions, lengths,
-    slots, sampling parameters, block-table rows of full width); a step copies the new values
+    slots, sampling parameters, block-table rows as wide as the bucket needs); a step copies the new values
     in and replays.  Nothing in the graph depends on a host-side number: the attention grid is
     fixed by the batch size and the bucket, key ranges are derived on the device from the lengths.
     """
@@ -242,7 +242,8 @@ class _DecodeGraph:
     def __init__(self, runner: "ModelRunner", R: int, length_bucket: int):
         self.runner, self.R = runner, R
         cache = runner.cache
-        self.width = cache.max_blocks
+        # no request of this graph is longer than the bucket: its tables need no more columns
+        self.width = min(cache.max_blocks, -(-length_bucket // cache.page_size))
         G = len(cache.groups)
         names = ["token_ids", "positions", "req_of_token", "kv_len", "slots", "logit_rows", "temps", "uniforms"]
         self.off, total = {}, 0

@@ -26,6 +26,9 @@ from ..weights.loader import TensorSpec
 from .base import MIXERS, KVCacheSpec, LayerCache, Mixer, PositionEncoding, StepContext
 
 
+POSITION_PREFIX = "position."
+
+
 class PagedAttention(Mixer):
     def __init__(
         self,
@@ -58,6 +61,8 @@ class PagedAttention(Mixer):
                 TensorSpec("v_proj.weight", (self.kv_size, self.hidden_size)),
             ]
         specs.append(TensorSpec("o_proj.weight", (self.hidden_size, self.q_size)))
+        if self.position is not None:     # a position encoding with tensors of its own keeps them under "position."
+            specs += [s.with_prefix(POSITION_PREFIX) for s in self.position.tensor_specs()]
         return specs
 
     def cache_spec(self):
@@ -73,7 +78,8 @@ class PagedAttention(Mixer):
         self.w_qkv = torch.cat([m.to(common) for m in mats], dim=0).contiguous()
         self.w_o = tensors["o_proj.weight"]
         if self.position is not None:
-            self.position.load({}, dtype, device)
+            own = {n[len(POSITION_PREFIX):]: t for n, t in tensors.items() if n.startswith(POSITION_PREFIX)}
+            self.position.load(own, dtype, device)
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
         T = h.shape[0]

@@ -275,3 +275,161 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         got = torch.cat(out[r])
         assert got.shape == want[r].shape
         assert (got - want[r]).abs().max() < 3e-5 * want[r].abs().max().clamp(min=1), r
+
+
+# ------------------------------------------------------------------ a second toy: routing and another position scheme
+def register_routed_toy():
+    """A feed-forward that routes every token to one of several small experts (router logits in
+    float32, the largest wins, lowest index among equals), and a position encoding that is no
+    rotation: a learned table added to queries and keys.  Both defined here, registered by name,
+    and chosen layer by layer: layer 0 routes, layer 1 has the ordinary gated feed-forward."""
+    from photon_infer_amd import register_architecture
+    from photon_infer_amd.parts import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, FeedForward, LMHead,
+                                        ModelSpec, PositionEncoding, RunEntry, TokenEmbedding)
+    from photon_infer_amd.weights import TensorSpec
+
+    class RoutedExperts(FeedForward):
+        def __init__(self, hidden_size, expert_size, num_experts, output_scale):
+            self.D, self.I, self.E, self.scale = hidden_size, expert_size, num_experts, output_scale
+
+        def tensor_specs(self):
+            specs = [TensorSpec("router.weight", (self.E, self.D))]
+            for e in range(self.E):
+                specs += [TensorSpec(f"experts.{e}.up.weight", (self.I, self.D)), TensorSpec(f"experts.{e}.down.weight", (self.D, self.I))]
+            return specs
+
+        def load(self, tensors, dtype, device):
+            super().load(tensors, dtype, device)
+            self.router = tensors["router.weight"].float()
+            self.up = [tensors[f"experts.{e}.up.weight"].float() for e in range(self.E)]
+            self.down = [tensors[f"experts.{e}.down.weight"].float() for e in range(self.E)]
+
+        def forward(self, h, x, ctx):
+            hf = h.float()
+            choice = (hf @ self.router.t()).argmax(dim=-1)          # float32 logits; argmax takes the lowest index among equals
+            for e in range(self.E):
+                rows = (choice == e).nonzero().flatten()
+                if rows.numel():
+                    x[rows] += self.scale * (torch.relu(hf[rows] @ self.up[e].t()) @ self.down[e].t())
+
+    FEED_FORWARDS.register("routed_experts", RoutedExperts)
+
+    class AddedPositions(PositionEncoding):
+        """q and k of the token at position p get table[p] added, the same vector for every head."""
+
+        def __init__(self, head_dim, max_positions):
+            self.head_dim, self.max_positions = head_dim, max_positions
+
+        def tensor_specs(self):
+            return [TensorSpec("table", (self.max_positions, self.head_dim))]
+
+        def load(self, tensors, dtype, device):
+            super().load(tensors, dtype, device)
+            self.table = tensors["table"].float()
+
+        def apply(self, q, k, ctx):
+            add = self.table[ctx.positions.long()]                  # [T, head_dim]
+            for t in (q, k):
+                if t is not None:
+                    v = t.view(t.shape[0], -1, self.head_dim)
+                    v += add[:, None, :].to(t.dtype)
+
+    POSITION_ENCODINGS.register("added_positions", AddedPositions)
+
+    @dataclasses.dataclass(frozen=True)
+    class RoutedConfig:
+        architecture: str
+        width: int
+        vocab: int
+        heads: int
+        experts: int
+        expert_width: int
+        expert_scale: float
+        norm_eps: float
+        torch_dtype: str = "float32"
+
+        @classmethod
+        def from_dict(cls, raw, where="config.json"):
+            return cls(raw["architectures"][0], raw["width"], raw["vocab"], raw["heads"], raw["experts"], raw["expert_width"],
+                       raw["expert_scale"], raw["norm_eps"], raw.get("torch_dtype", "float32"))
+
+        def to_dict(self):
+            d = dataclasses.asdict(self)
+            d["architectures"] = [d.pop("architecture")]
+            return d
+
+    def build(cfg):
+        D, hd = cfg.width, cfg.width // cfg.heads
+        norm = lambda: NORMS.make("rmsnorm", dim=D, eps=cfg.norm_eps)
+
+        def block(ffn):
+            # every layer has a position table of its own: the part is given under the mixer's prefix
+            mixer = MIXERS.make("attention", hidden_size=D, num_heads=cfg.heads, num_kv_heads=cfg.heads, head_dim=hd,
+                                position=POSITION_ENCODINGS.make("added_positions", head_dim=hd, max_positions=40))
+            return BLOCKS.make("prenorm", norm1=("n1.", norm()), mixer=("attn.", mixer), norm2=("n2.", norm()), ffn=("ffn.", ffn))
+        layers = [("l0.", block(FEED_FORWARDS.make("routed_experts", hidden_size=D, expert_size=cfg.expert_width,
+                                                    num_experts=cfg.experts, output_scale=cfg.expert_scale))),
+                  ("l1.", block(FEED_FORWARDS.make("swiglu", hidden_size=D, intermediate_size=3 * D)))]
+        return ModelSpec(hidden_size=D, vocab_size=cfg.vocab, max_positions=40, embedding=("emb.", TokenEmbedding(cfg.vocab, D)),
+                         layers=layers, run_order=[RunEntry(0), RunEntry(1)], final_norm=("norm.", norm()),
+                         head=("head.", LMHead(cfg.vocab, D, tied=True)))
+
+    register_architecture("RoutedToyForCausalLM", RoutedConfig, build)
+    return RoutedConfig
+
+
+def plain_routed_toy(cfg, W, toks):
+    D, nh, S, eps = cfg["width"], cfg["heads"], len(toks), cfg["norm_eps"]
+    hd = D // nh
+    x = P.embedding(W["emb.weight"], toks)
+    for l in ("l0.", "l1."):
+        h = P.rmsnorm(x, W[l + "n1.weight"], eps)
+        add = W[l + "attn.position.table"][:S][:, None, :]
+        q = P.linear(h, W[l + "attn.q_proj.weight"]).reshape(S, nh, hd) + add
+        k = P.linear(h, W[l + "attn.k_proj.weight"]).reshape(S, nh, hd) + add
+        v = P.linear(h, W[l + "attn.v_proj.weight"]).reshape(S, nh, hd)
+        x = x + P.linear(P.attention(q, k, v, 1 / math.sqrt(hd)).reshape(S, D), W[l + "attn.o_proj.weight"])
+        h = P.rmsnorm(x, W[l + "n2.weight"], eps)
+        if l == "l0.":
+            choice = P.linear(h, W[l + "ffn.router.weight"]).argmax(dim=-1)
+            out = torch.zeros_like(x)
+            for t in range(S):
+                e = int(choice[t])
+                out[t] = cfg["expert_scale"] * P.linear(torch.relu(P.linear(h[t:t + 1], W[f"{l}ffn.experts.{e}.up.weight"])),
+                                                         W[f"{l}ffn.experts.{e}.down.weight"])[0]
+            x = x + out
+        else:
+            x = x + P.linear(P.swiglu(P.linear(h, W[l + "ffn.gate_proj.weight"]), P.linear(h, W[l + "ffn.up_proj.weight"])),
+                             W[l + "ffn.down_proj.weight"])
+    return P.linear(P.rmsnorm(x, W["norm.weight"], eps), W["emb.weight"]), None
+
+
+def test_toy_routed_feed_forward_and_added_positions(tmp_path):
+    """Registered from here: a feed-forward with routing and a position encoding that is not a
+    rotation; built from config.json, stepped whole and in portions beside another request."""
+    from photon_infer_amd import write_random_model
+    from photon_infer_amd.engine import EngineOptions, ModelRunner, StepEntry
+    RoutedConfig = register_routed_toy()
+    cfg = RoutedConfig("RoutedToyForCausalLM", width=32, vocab=83, heads=2, experts=3, expert_width=56, expert_scale=0.7, norm_eps=1e-6)
+    d = write_random_model(cfg, str(tmp_path / "routed"), seed=5, std=0.2, norm_init="uniform", dtype="float32")
+    raw, W = P.read_model_folder(d)
+    assert "l0.attn.position.table" in W and "l1.attn.position.table" in W and "l0.ffn.experts.2.down.weight" in W
+    runner = ModelRunner(d, EngineOptions(dtype="float32", block_size=4, num_blocks=20, max_batch=2))
+    seqs = {"a": random_tokens(26, 83, 4), "b": random_tokens(19, 83, 5)}
+    want = {k: plain_routed_toy(raw, W, v)[0] for k, v in seqs.items()}
+    runner.admit("a")
+    got = runner.step([StepEntry("a", seqs["a"], list(range(26)))]).cpu()
+    assert (got - want["a"]).abs().max() < 3e-5 * want["a"].abs().max().clamp(min=1)
+    runner.release("a")
+    runner.admit("a"); runner.admit("b")
+    out, pos = {"a": [], "b": []}, {"a": 0, "b": 0}
+    for na, nb in [(3, 2), (1, 9), (12, 1), (10, 1), (0, 6)]:
+        entries = [StepEntry(r, seqs[r][pos[r]:pos[r] + n], list(range(n))) for r, n in (("a", na), ("b", nb)) if n]
+        logits = runner.step(entries).cpu()
+        i = 0
+        for e in entries:
+            out[e.rid].append(logits[i:i + len(e.tokens)]); i += len(e.tokens); pos[e.rid] += len(e.tokens)
+    for r in ("a", "b"):
+        got = torch.cat(out[r])
+        assert got.shape == want[r].shape
+        assert (got - want[r]).abs().max() < 3e-5 * want[r].abs().max().clamp(min=1), r
