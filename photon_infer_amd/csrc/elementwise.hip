@@ -246,6 +246,107 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
   }
 }
 
+// The same for the common case, many tokens at a time (prompts): bfloat16 tensors (no pieces),
+// rotation over the whole head with halves paired, head size a multiple of 16.  Every memory
+// access is wide: a thread turns 8 features and their 8 partners of one (token, head) (16-byte
+// loads and stores, in place for queries, into the page for keys); for values a thread takes
+// one feature of four consecutive tokens and, when the four are neighbours in one page,
+// stores them with one 8-byte write into the transposed page.
+__global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
+    bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k, long k_stride, const bf16_t* __restrict__ v,
+    long v_stride, const int* __restrict__ positions, const int* __restrict__ req_of_token, const float* __restrict__ table,
+    int rotate, int T, int nh, int nkv_write, int nkv, int hd, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
+    const int* __restrict__ block_table, int table_width, int page_size, long num_pages, long rot_items) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  const int units = hd / 16, heads = nh + nkv_write;
+  if (idx < rot_items) {
+    const int unit = (int)(idx % units), head = (int)((idx / units) % heads);
+    const long t = idx / ((long)units * heads);
+    const int d = unit * 8;                      // features d .. d + 7 and their partners at + hd / 2
+    const bf16_t* src;
+    bf16_t* dst;
+    if (head < nh) {
+      dst = q + t * q_stride + (long)head * hd;
+      src = dst;
+    } else {
+      const int g = head - nh, pos = positions[t], blk = pos / page_size;
+      if (blk >= table_width) return;
+      const long page = block_table[(long)req_of_token[t] * table_width + blk];
+      if (page < 0 || page >= num_pages) return;   // the host checks tables; never write outside the pool
+      src = k + t * k_stride + (long)g * hd;
+      dst = k_cache + ((page * nkv + g) * page_size + (pos % page_size)) * hd;
+    }
+    if (!rotate && dst == src) return;
+    const uint4 lo = *reinterpret_cast<const uint4*>(src + d), hi = *reinterpret_cast<const uint4*>(src + d + hd / 2);
+    uint4 out_lo = lo, out_hi = hi;
+    if (rotate) {
+      const float* c = table + t * hd + d;
+      const float* sn = c + hd / 2;
+      typedef float quad_t __attribute__((ext_vector_type(4)));
+      const quad_t c0 = *reinterpret_cast<const quad_t*>(c), c1 = *reinterpret_cast<const quad_t*>(c + 4);
+      const quad_t s0 = *reinterpret_cast<const quad_t*>(sn), s1 = *reinterpret_cast<const quad_t*>(sn + 4);
+      const uint32_t* lw = reinterpret_cast<const uint32_t*>(&lo);
+      const uint32_t* hw = reinterpret_cast<const uint32_t*>(&hi);
+      uint32_t ol[4], oh[4];
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {              // two features per 32-bit word
+        float a[2] = {__uint_as_float(lw[w] << 16), __uint_as_float(lw[w] & 0xffff0000u)};
+        float b[2] = {__uint_as_float(hw[w] << 16), __uint_as_float(hw[w] & 0xffff0000u)};
+        float rl[2], rh[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const int i = 2 * w + e;
+          const float cc = i < 4 ? c0[i] : c1[i - 4], ss = i < 4 ? s0[i] : s1[i - 4];
+          rl[e] = a[e] * cc - b[e] * ss;
+          rh[e] = a[e] * ss + b[e] * cc;
+        }
+        ol[w] = f32x2_to_bf16x2_bits(rl[0], rl[1]);
+        oh[w] = f32x2_to_bf16x2_bits(rh[0], rh[1]);
+      }
+      out_lo = make_uint4(ol[0], ol[1], ol[2], ol[3]);
+      out_hi = make_uint4(oh[0], oh[1], oh[2], oh[3]);
+    }
+    *reinterpret_cast<uint4*>(dst + d) = out_lo;
+    *reinterpret_cast<uint4*>(dst + d + hd / 2) = out_hi;
+    return;
+  }
+  // values: (four tokens, kv head, feature)
+  const long j = idx - rot_items;
+  const int d = (int)(j % hd), g = (int)((j / hd) % nkv);
+  const long t0 = (j / ((long)hd * nkv)) * 4;
+  if (nkv_write == 0 || t0 >= T) return;
+  const int n = (int)min((long)4, T - t0);
+  uint16_t val[4];
+  int pos[4], req[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const long t = t0 + (i < n ? i : 0);
+    val[i] = *reinterpret_cast<const uint16_t*>(v + t * v_stride + (long)g * hd + d);
+    pos[i] = positions[t];
+    req[i] = req_of_token[t];
+  }
+  const bool together = n == 4 && pos[0] % 4 == 0 && req[3] == req[0] && req[1] == req[0] && req[2] == req[0] &&
+                        pos[1] == pos[0] + 1 && pos[2] == pos[0] + 2 && pos[3] == pos[0] + 3;
+  if (together) {                                  // page sizes are multiples of 4 here: one page, four slots in a row
+    const int blk = pos[0] / page_size;
+    if (blk >= table_width) return;
+    const long page = block_table[(long)req[0] * table_width + blk];
+    if (page < 0 || page >= num_pages) return;
+    uint2 w;
+    w.x = (uint32_t)val[0] | ((uint32_t)val[1] << 16);
+    w.y = (uint32_t)val[2] | ((uint32_t)val[3] << 16);
+    *reinterpret_cast<uint2*>(v_cache + (page * nkv + g) * (long)page_size * hd + (long)d * page_size + pos[0] % page_size) = w;
+    return;
+  }
+  for (int i = 0; i < n; ++i) {
+    const int blk = pos[i] / page_size;
+    if (blk >= table_width) continue;
+    const long page = block_table[(long)req[i] * table_width + blk];
+    if (page < 0 || page >= num_pages) continue;
+    reinterpret_cast<uint16_t*>(v_cache)[(page * nkv + g) * (long)page_size * hd + (long)d * page_size + pos[i] % page_size] = val[i];
+  }
+}
+
 extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride,
                                 int dtype, const int* positions, const int* req_of_token, const float* table,
                                 int rotary_dim, int interleaved, int T, int nh, int nkv, int hd, int write_kv,
@@ -262,6 +363,23 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
   }
   const int heads = nh + (write_kv ? 2 * nkv : 0);
   if (T == 0 || heads == 0) return 0;
+  // many bfloat16 tokens with the usual rotation: the kernel with wide accesses
+  const bool usual = rotary_dim == 0 || (rotary_dim == hd && !interleaved);
+  const bool aligned = hd % 16 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && (!table || (uintptr_t)table % 16 == 0) &&
+                       (!write_kv || (k_stride % 8 == 0 && ((uintptr_t)k % 16 == 0) && ((uintptr_t)k_cache % 16 == 0) &&
+                                      ((uintptr_t)v_cache % 8 == 0) && page_size % 4 == 0));
+  if (dtype == PI_BF16 && !part && usual && aligned && T >= 16) {
+    const int nkv_w = write_kv ? nkv : 0;
+    const long rot_items = (long)T * (nh + nkv_w) * (hd / 16);
+    const long v_items = write_kv ? (long)((T + 3) / 4) * nkv * hd : 0;
+    const long blocks = (rot_items + v_items + 255) / 256;
+    PI_REQUIRE(blocks < 2147483647L, "rope_kv_write: too many tokens (%d)", T);
+    hipLaunchKernelGGL(rope_kv_write_wide_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (bf16_t*)q, q_stride,
+                       (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, positions, req_of_token, table,
+                       rotary_dim > 0 ? 1 : 0, T, nh, nkv_w, nkv, hd, (bf16_t*)k_cache, (bf16_t*)v_cache, block_table,
+                       table_width, page_size, num_pages, rot_items);
+    return pi_check_launch("rope_kv_write_wide");
+  }
   PI_REQUIRE(heads <= 65535, "rope_kv_write: too many heads (%d)", heads);
   const dim3 grid(T, (heads + 3) / 4), block(256);
   const int nkv_write = write_kv ? nkv : 0;
