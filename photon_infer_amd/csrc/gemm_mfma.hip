@@ -9,7 +9,7 @@
 // the same (row, feature) sit 16 lanes apart; one row swap brings them together and
 // silu(gate) * up is stored directly.
 //
-// Any M and N (edges are zero-filled on load and skipped on store); K must be a multiple of
+// Any M and N (edges read zeros and are skipped on store); K must be a multiple of
 // 8 and row strides multiples of 8 so that 16-byte loads stay aligned.  Each output row
 // accumulates over k in the same order whatever the other rows are.
 #include "mfma.h"
@@ -29,6 +29,21 @@ enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACCUM = 2, EPI_SWIGLU = 3 };
 __device__ inline float silu_mul(float g, float u) {
   return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g)) * u;
 }
+
+// Global loads go through buffer descriptors: a scalar base (the block's first row at its first
+// k), a byte length, and per-lane 32-bit offsets.  An offset at or beyond the length reads
+// zeros, which is how rows beyond the matrix and k beyond the range are filled, without a branch.
+#define PI_OUT_OF_RANGE 0x7ffffff0u
+#if defined(__HIP_DEVICE_COMPILE__)
+__device__ inline __amdgpu_buffer_rsrc_t operand_descriptor(const bf16_t* base, long bytes) {
+  // made scalar by hand so that the loads take the descriptor from scalar registers
+  const uint64_t v = reinterpret_cast<uint64_t>(base);
+  const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
+  const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+  void* p = reinterpret_cast<void*>((static_cast<uint64_t>(hi) << 32) | lo);
+  return __builtin_amdgcn_make_buffer_rsrc(p, 0, __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000);
+}
+#endif
 
 template <int EPI>
 __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ A, long lda,
@@ -64,22 +79,37 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
   // that sixteen lanes land on 64 distinct LDS banks with rows 144 bytes apart)
   const int lgrp = tid / 8, lchunk = tid % 8;
   const int lrow = (lgrp / 16) * 16 + ((lgrp / 8) % 2) * 4 + (lgrp % 8) / 2 + 8 * (lgrp % 2);
-  uint4 ra[4], rw[4];
+  const int a_rows = (int)min((long)BM, M - m0), w_rows = (int)min((long)BN, N - n0);
+#if defined(__HIP_DEVICE_COMPILE__)
+  const __amdgpu_buffer_rsrc_t a_src = operand_descriptor(A + m0 * lda + k_lo, ((long)(a_rows - 1) * lda + (k_hi - k_lo)) * 2);
+  const __amdgpu_buffer_rsrc_t w_src = operand_descriptor(W + n0 * ldw + k_lo, ((long)(w_rows - 1) * ldw + (k_hi - k_lo)) * 2);
+#endif
+  unsigned a_off[4], w_off[4];
+#pragma unroll
+  for (int p = 0; p < 4; ++p) {
+    const int row = lrow + 32 * p;
+    a_off[p] = row < a_rows ? (unsigned)(row * (int)lda + lchunk * 8) * 2u : PI_OUT_OF_RANGE;
+    w_off[p] = row < w_rows ? (unsigned)(row * (int)ldw + lchunk * 8) * 2u : PI_OUT_OF_RANGE;
+  }
+  u32x4_t ra[4], rw[4];
   auto load_slab = [&](int k0) {
-    const int k = k0 + lchunk * 8;
+    // k0 is relative to k_lo; this lane's 8 k of the slab may lie beyond the range (last slab)
+    const unsigned kb = (unsigned)k0 * 2u;
+    const bool k_in = k0 + lchunk * 8 < k_hi - k_lo;
+#if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
-      const long m = m0 + lrow + 32 * p, n = n0 + lrow + 32 * p;
-      ra[p] = (m < M && k < k_hi) ? *reinterpret_cast<const uint4*>(A + m * lda + k) : make_uint4(0, 0, 0, 0);
-      rw[p] = (n < N && k < k_hi) ? *reinterpret_cast<const uint4*>(W + n * ldw + k) : make_uint4(0, 0, 0, 0);
+      ra[p] = __builtin_amdgcn_raw_buffer_load_b128(a_src, k_in ? a_off[p] + kb : PI_OUT_OF_RANGE, 0, 0);
+      rw[p] = __builtin_amdgcn_raw_buffer_load_b128(w_src, k_in ? w_off[p] + kb : PI_OUT_OF_RANGE, 0, 0);
     }
+#endif
   };
   auto store_slab = [&](int buf) {
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
       const int off = (lrow + 32 * p) * LDS_ROW + lchunk * 8;
-      *reinterpret_cast<uint4*>(As + buf * TILE_ELEMS + off) = ra[p];
-      *reinterpret_cast<uint4*>(Ws + buf * TILE_ELEMS + off) = rw[p];
+      *reinterpret_cast<u32x4_t*>(As + buf * TILE_ELEMS + off) = ra[p];
+      *reinterpret_cast<u32x4_t*>(Ws + buf * TILE_ELEMS + off) = rw[p];
     }
   };
 
@@ -92,7 +122,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   const int slabs = (k_hi - k_lo + BK - 1) / BK;
-  load_slab(k_lo);
+  load_slab(0);
   store_slab(0);
   __syncthreads();
   // 32 x 32 x 16 instruction: a lane reads row lane % 32, 16 bytes at k = (lane / 32) * 8; with
@@ -100,7 +130,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
   const int frow = lane % 32, fk = (lane / 32) * 8;
   for (int s = 0; s < slabs; ++s) {
     const int buf = s & 1;
-    if (s + 1 < slabs) load_slab(k_lo + (s + 1) * BK);
+    if (s + 1 < slabs) load_slab((s + 1) * BK);
     const uint16_t* a_base = As + buf * TILE_ELEMS + (wm * 64 + frow) * LDS_ROW + fk;
     const uint16_t* w_base = Ws + buf * TILE_ELEMS + (wn * 64 + frow) * LDS_ROW + fk;
 #pragma unroll
@@ -201,17 +231,8 @@ __global__ __launch_bounds__(256) void gemm_mfma_big_kernel(void* __restrict__ C
   const int lrow = (lgrp / 16) * 16 + ((lgrp / 8) % 2) * 4 + (lgrp % 8) / 2 + 8 * (lgrp % 2);
   const int a_rows = (int)min((long)GM, M - m0), w_rows = (int)min((long)GN, N - n0);
 #if defined(__HIP_DEVICE_COMPILE__)
-  // descriptors: base of the block's rows at k_lo, length up to the end of its last row; built
-  // from values made scalar by hand so that the loads take them from scalar registers
-  auto descriptor = [](const bf16_t* base, long bytes) {
-    const uint64_t v = reinterpret_cast<uint64_t>(base);
-    const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
-    const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
-    void* p = reinterpret_cast<void*>((static_cast<uint64_t>(hi) << 32) | lo);
-    return __builtin_amdgcn_make_buffer_rsrc(p, 0, __builtin_amdgcn_readfirstlane((int)bytes), 0x00020000);
-  };
-  const __amdgpu_buffer_rsrc_t a_src = descriptor(A + m0 * lda + k_lo, ((long)(a_rows - 1) * lda + (k_hi - k_lo)) * 2);
-  const __amdgpu_buffer_rsrc_t w_src = descriptor(W + n0 * ldw + k_lo, ((long)(w_rows - 1) * ldw + (k_hi - k_lo)) * 2);
+  const __amdgpu_buffer_rsrc_t a_src = operand_descriptor(A + m0 * lda + k_lo, ((long)(a_rows - 1) * lda + (k_hi - k_lo)) * 2);
+  const __amdgpu_buffer_rsrc_t w_src = operand_descriptor(W + n0 * ldw + k_lo, ((long)(w_rows - 1) * ldw + (k_hi - k_lo)) * 2);
 #endif
   unsigned a_off[8], w_off[8];
 #pragma unroll
@@ -363,8 +384,7 @@ static int launch(void* C, long ldc, const void* A, long lda, const void* W, lon
   kps = ((kps + BK - 1) / BK) * BK;
   splits = ceil_div(K, kps);
   const long big_tiles = (long)ceil_div(M, GM) * ceil_div(N, GN);
-  if (big_tiles * splits >= BIG_MIN_TILES && big_tiles < 2147483647L && ldc < (1L << 23) && K % BK == 0 &&
-      256 * lda < (1L << 30) && 256 * ldw < (1L << 30)) {
+  if (big_tiles * splits >= BIG_MIN_TILES && big_tiles < 2147483647L && ldc < (1L << 23) && K % BK == 0) {
     static bool big_configured = false;
     if (!big_configured) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma_big_kernel<EPI>),
@@ -399,6 +419,7 @@ extern "C" int pi_gemm_mfma(void* C, int epilogue, long ldc, const void* A, long
   PI_REQUIRE(splits >= 1 && splits <= 64 && (splits == 1 || (epilogue == EPI_F32 && ldc == N)),
              "gemm_mfma: a k-split (%d) needs the float32 store into a [splits, M, N] workspace", splits);
   PI_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gemm_mfma: K (%d) and row strides (%ld, %ld) must be multiples of 8", K, lda, ldw);
+  PI_REQUIRE(256 * lda < (1L << 29) && 256 * ldw < (1L << 29), "gemm_mfma: row strides (%ld, %ld) are too long for 32-bit offsets inside a tile", lda, ldw);
   PI_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_mfma: operands must be 16-byte aligned");
   PI_REQUIRE(epilogue != EPI_SWIGLU || N % 32 == 0, "gemm_mfma: the SwiGLU epilogue needs N (%d) to be a multiple of 32", N);
   PI_REQUIRE((long)ceil_div(M, BM) * ceil_div(N, BN) < 2147483647L, "gemm_mfma: too many tiles");
