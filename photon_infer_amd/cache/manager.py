@@ -13,33 +13,50 @@ Reference: src/runtime/kv_cache_manager.cpp (one pool, same block id in all laye
 * every live request owns a *slot*: the row of its block tables and the index of its
   fixed-size state, if any mixer keeps one.
 
-The manager is host-side bookkeeping only; it never touches device memory.
+The manager is host-side bookkeeping only; it never touches device memory.  The bookkeeping
+itself is native (``csrc/runtime/cache.cpp``): this class maps request ids to slots, turns
+status codes into exceptions, and hands out numpy views of the native block tables.
 """
 from __future__ import annotations
 
-from dataclasses import dataclass, field
+import ctypes
 from typing import Dict, Hashable, List, Optional, Sequence
 
 import numpy as np
 
 from ..errors import CacheError, OutOfPagesError
-from .pages import PagePool
+from . import _native
 
 
-@dataclass
+class _GroupPool:
+    """What callers may ask about a group's page pool."""
+
+    def __init__(self, manager: "CacheManager", index: int, num_pages: int):
+        self._m, self._g, self.num_pages = manager, index, num_pages
+
+    @property
+    def num_free(self) -> int:
+        return self._m._lib.pi_cache_free_pages(self._m._h, self._g)
+
+    @property
+    def num_allocated(self) -> int:
+        return self.num_pages - self.num_free
+
+    def is_allocated(self, page: int) -> bool:
+        return bool(self._m._lib.pi_cache_page_allocated(self._m._h, self._g, int(page)))
+
+
 class _Group:
-    window: Optional[int]
-    pool: PagePool
-    table: np.ndarray                      # [max_slots, max_blocks] int32, -1 = no page
-    next_block: list                       # [max_slots] blocks ever allocated (index of the next one)
-    first_block: list                      # [max_slots] first block still held
+    """A view of one cache group: its window, pool and block tables (numpy views of native memory)."""
 
-
-@dataclass
-class _Request:
-    slot: int
-    length: int = 0     # tokens whose keys are in the cache
-    reserved: int = 0   # tokens that pages are held for (>= length)
+    def __init__(self, manager: "CacheManager", index: int, window: Optional[int], num_pages: int):
+        lib, h = manager._lib, manager._h
+        self.window = window
+        self.pool = _GroupPool(manager, index, num_pages)
+        shape = (manager.max_slots, manager.max_blocks)
+        self.table = np.ctypeslib.as_array(lib.pi_cache_table(h, index), shape=shape)          # -1 = no page
+        self.next_block = np.ctypeslib.as_array(lib.pi_cache_next_block(h, index), shape=(manager.max_slots,))
+        self.first_block = np.ctypeslib.as_array(lib.pi_cache_first_block(h, index), shape=(manager.max_slots,))
 
 
 class CacheManager:
@@ -56,167 +73,146 @@ class CacheManager:
         counts = [num_pages] * len(windows) if isinstance(num_pages, int) else list(num_pages)
         if len(counts) != len(windows):
             raise CacheError(f"{len(windows)} cache groups but {len(counts)} pool sizes")
-        self.groups: List[_Group] = [
-            _Group(w, PagePool(n), np.full((self.max_slots, self.max_blocks), -1, np.int32),
-                   [0] * self.max_slots, [0] * self.max_slots)
-            for w, n in zip(windows, counts)
-        ]
-        self._requests: Dict[Hashable, _Request] = {}
-        self._free_slots: List[int] = list(range(self.max_slots - 1, -1, -1))
+        if any(int(n) <= 0 for n in counts):
+            raise CacheError(f"a page pool needs at least one page, got {counts}")
+        self._lib = _native.lib()
+        self._h = self._lib.pi_cache_create(len(windows), _native.int_array(-1 if w is None else int(w) for w in windows),
+                                            self.page_size, _native.int_array(int(n) for n in counts), self.max_slots,
+                                            self.max_model_len)
+        if not self._h:
+            raise CacheError("the native cache manager refused its sizes")
+        self.groups: List[_Group] = [_Group(self, i, w, int(n)) for i, (w, n) in enumerate(zip(windows, counts))]
+        self._lengths = np.ctypeslib.as_array(self._lib.pi_cache_lengths(self._h), shape=(self.max_slots,))
+        self._slots: Dict[Hashable, int] = {}
+        self._need = _native.int_array([0] * len(self.groups))
+
+    def __del__(self):
+        h, self._h = getattr(self, "_h", None), None
+        if h:
+            self.groups = []          # the views point into native memory
+            self._lib.pi_cache_destroy(h)
+
+    def _fail(self, status: int, rid: Hashable = None):
+        msg = self._lib.pi_cache_error(self._h).decode()
+        if rid is not None:
+            msg = f"request {rid!r}: {msg}"
+        raise (OutOfPagesError if status == _native.OUT_OF_PAGES else CacheError)(msg)
 
     # ------------------------------------------------------------------ queries
     def __contains__(self, rid: Hashable) -> bool:
-        return rid in self._requests
+        return rid in self._slots
 
     @property
     def num_live(self) -> int:
-        return len(self._requests)
+        return len(self._slots)
 
     @property
     def free_slots(self) -> int:
-        return len(self._free_slots)
+        return self._lib.pi_cache_free_slots(self._h)
 
     def free_pages(self, group: int = 0) -> int:
-        return self.groups[group].pool.num_free
+        return self._lib.pi_cache_free_pages(self._h, group)
 
-    def _req(self, rid: Hashable) -> _Request:
+    def slot(self, rid: Hashable) -> int:
         try:
-            return self._requests[rid]
+            return self._slots[rid]
         except KeyError:
             raise CacheError(f"request {rid!r} is not live in the cache") from None
 
-    def slot(self, rid: Hashable) -> int:
-        return self._req(rid).slot
-
     def length(self, rid: Hashable) -> int:
-        return self._req(rid).length
+        return int(self._lengths[self.slot(rid)])
 
     def pages_needed(self, rid: Optional[Hashable], new_tokens: int) -> List[int]:
         """Pages each group must still hand out for ``rid`` to grow by ``new_tokens``
-        (``rid`` None: a request that is not admitted yet)."""
-        r = self._requests.get(rid) if rid is not None else None
-        target = (r.length if r else 0) + new_tokens
-        blocks = -(-target // self.page_size)
-        if r is None:
-            return [blocks] * len(self.groups)
-        slot = r.slot
-        return [max(0, blocks - g.next_block[slot]) for g in self.groups]
+        (``rid`` None or unknown: a request that is not admitted yet)."""
+        slot = self._slots.get(rid, -1) if rid is not None else -1
+        self._lib.pi_cache_pages_needed(self._h, slot, int(new_tokens), self._need)
+        return list(self._need[:len(self.groups)])
 
     def can_reserve(self, rid: Optional[Hashable], new_tokens: int, held_back: Sequence[int] | None = None) -> bool:
         """Whether ``reserve`` would succeed; ``held_back[g]`` pages of group g count as taken."""
-        need = self.pages_needed(rid, new_tokens)
-        return all(n <= g.pool.num_free - (held_back[i] if held_back else 0)
-                   for i, (n, g) in enumerate(zip(need, self.groups)))
+        slot = self._slots.get(rid, -1) if rid is not None else -1
+        held = _native.int_array(held_back) if held_back else None
+        return bool(self._lib.pi_cache_can_reserve(self._h, slot, int(new_tokens), held))
 
     # ------------------------------------------------------------------ life cycle
     def admit(self, rid: Hashable) -> int:
         """Give ``rid`` a slot.  Its block-table rows start empty."""
-        if rid in self._requests:
+        if rid in self._slots:
             raise CacheError(f"request {rid!r} is already live in the cache")
-        if not self._free_slots:
-            raise CacheError(f"no free slot: {self.max_slots} requests are live")
-        slot = self._free_slots.pop()
-        self._requests[rid] = _Request(slot)
+        slot = self._lib.pi_cache_admit(self._h)
+        if slot < 0:
+            self._fail(_native.MISUSE)
+        self._slots[rid] = slot
         return slot
 
     def reserve(self, rid: Hashable, new_tokens: int) -> None:
         """Hold pages for positions ``length .. length + new_tokens - 1`` in every group,
         all or nothing (OutOfPagesError leaves everything as it was)."""
-        r = self._req(rid)
-        if new_tokens < 0:
-            raise CacheError(f"cannot reserve {new_tokens} tokens")
-        target = r.length + new_tokens
-        if target > self.max_model_len:
-            raise CacheError(f"request {rid!r} would hold {target} tokens; the limit is {self.max_model_len}")
-        need = self.pages_needed(rid, new_tokens)
-        for i, (n, g) in enumerate(zip(need, self.groups)):
-            if n > g.pool.num_free:
-                raise OutOfPagesError(
-                    f"request {rid!r} needs {n} more pages in cache group {i}, {g.pool.num_free} are free")
-        for n, g in zip(need, self.groups):
-            if n:
-                pages = g.pool.allocate(n)
-                b = int(g.next_block[r.slot])
-                g.table[r.slot, b:b + n] = pages
-                g.next_block[r.slot] = b + n
-        r.reserved = max(r.reserved, target)
+        status = self._lib.pi_cache_reserve(self._h, self.slot(rid), int(new_tokens))
+        if status:
+            self._fail(status, rid)
 
     def commit(self, rid: Hashable, new_tokens: int) -> None:
         """The step wrote ``new_tokens`` more keys: advance the length and give back the
         pages that every window has passed."""
-        r = self._req(rid)
-        if r.length + new_tokens > r.reserved:
-            raise CacheError(
-                f"request {rid!r}: committing to {r.length + new_tokens} tokens but pages are held for {r.reserved}")
-        r.length += new_tokens
-        for g in self.groups:
-            if g.window is None:
-                continue
-            # the next query sits at position >= length and reads keys >= length - window + 1
-            first_needed = max(0, r.length - g.window + 1) // self.page_size
-            lo = int(g.first_block[r.slot])
-            hi = min(first_needed, int(g.next_block[r.slot]))
-            if hi > lo:
-                g.pool.free(int(p) for p in g.table[r.slot, lo:hi])
-                g.table[r.slot, lo:hi] = -1
-                g.first_block[r.slot] = hi
+        status = self._lib.pi_cache_commit(self._h, self.slot(rid), int(new_tokens))
+        if status:
+            self._fail(status, rid)
+
+    def reserve_step(self, slots: Sequence[int], new_tokens: Sequence[int]) -> None:
+        """Pages for a whole step, all or nothing: either every request of the step can grow
+        or nothing is taken (OutOfPagesError)."""
+        n = len(slots)
+        status = self._lib.pi_cache_reserve_many(self._h, _native.int_array(slots), _native.int_array(new_tokens), n)
+        if status:
+            self._fail(status)
+
+    def commit_step(self, slots: Sequence[int], new_tokens: Sequence[int]) -> None:
+        status = self._lib.pi_cache_commit_many(self._h, _native.int_array(slots), _native.int_array(new_tokens), len(slots))
+        if status:
+            self._fail(status)
 
     def release(self, rid: Hashable) -> int:
         """The request ended (or was preempted): give back its pages and its slot."""
-        r = self._req(rid)
-        for g in self.groups:
-            lo, hi = int(g.first_block[r.slot]), int(g.next_block[r.slot])
-            if hi > lo:
-                g.pool.free(int(p) for p in g.table[r.slot, lo:hi])
-            g.table[r.slot, :] = -1
-            g.next_block[r.slot] = 0
-            g.first_block[r.slot] = 0
-        del self._requests[rid]
-        self._free_slots.append(r.slot)
-        return r.slot
+        slot = self.slot(rid)
+        status = self._lib.pi_cache_release(self._h, slot)
+        if status:
+            self._fail(status, rid)
+        del self._slots[rid]
+        return slot
 
     def reset(self) -> None:
-        for rid in list(self._requests):
+        for rid in list(self._slots):
             self.release(rid)
 
     # ------------------------------------------------------------------ for the step function
     def table_rows(self, group: int, slots: Sequence[int], width: Optional[int] = None) -> np.ndarray:
-        """Block-table rows of ``slots`` (int32 [len(slots), width])."""
+        """Block-table rows of ``slots`` (int32 [len(slots), width], a copy)."""
         g = self.groups[group]
         w = self.max_blocks if width is None else width
         return g.table[np.asarray(slots, dtype=np.int64), :w]
 
+    def lengths_of(self, slots: Sequence[int]) -> np.ndarray:
+        """Cached tokens of ``slots`` (int32, a copy)."""
+        return self._lengths[np.asarray(slots, dtype=np.int64)]
+
     def blocks_in_use(self, slots: Sequence[int]) -> int:
         """Largest block index + 1 among ``slots`` over all groups."""
-        if not len(slots):
+        if not len(slots) or not self.groups:
             return 0
         idx = np.asarray(slots, dtype=np.int64)
-        return max(max(g.next_block[int(i)] for i in idx) for g in self.groups) if self.groups else 0
+        return int(max(g.next_block[idx].max() for g in self.groups))
 
     # ------------------------------------------------------------------ checks and numbers
     def check_invariants(self) -> None:
         """No page lost, none held twice: every allocated page appears exactly once in the
         tables of live requests and every page in a table is allocated."""
-        live_slots = {r.slot for r in self._requests.values()}
-        if len(live_slots) != len(self._requests) or live_slots & set(self._free_slots):
+        if len(set(self._slots.values())) != len(self._slots) or len(self._slots) + self.free_slots != self.max_slots:
             raise CacheError("slot bookkeeping is inconsistent")
-        if len(live_slots) + len(self._free_slots) != self.max_slots:
-            raise CacheError("a slot was lost")
-        for gi, g in enumerate(self.groups):
-            held: List[int] = []
-            for s in range(self.max_slots):
-                row = g.table[s]
-                pages = row[row >= 0]
-                if s not in live_slots and len(pages):
-                    raise CacheError(f"group {gi}: free slot {s} still holds pages")
-                lo, hi = int(g.first_block[s]), int(g.next_block[s])
-                if len(pages) != hi - lo or (hi > lo and (row[lo:hi] < 0).any()):
-                    raise CacheError(f"group {gi}: slot {s} table does not match its block range")
-                held += [int(p) for p in pages]
-            if len(held) != len(set(held)):
-                raise CacheError(f"group {gi}: a page is held twice")
-            if len(held) != g.pool.num_allocated or any(not g.pool.is_allocated(p) for p in held):
-                raise CacheError(f"group {gi}: {g.pool.num_allocated} pages allocated but {len(held)} in tables")
+        status = self._lib.pi_cache_check(self._h)
+        if status:
+            self._fail(status)
 
     def utilization(self, group: int = 0) -> float:
         g = self.groups[group]

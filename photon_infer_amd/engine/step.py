@@ -166,18 +166,12 @@ class ModelRunner:
         ops.attach_attention_plan(ctx, extra, views)
         return ctx
 
-    def _reserve(self, entries: Sequence[StepEntry]) -> None:
-        """Pages for the step's new tokens: refuse the whole step before taking any page."""
-        held = [0] * len(self.cache.groups)
-        for e in entries:
-            need = self.cache.pages_needed(e.rid, len(e.tokens))
-            held = [h + n for h, n in zip(held, need)]
-        for g, h in enumerate(held):
-            if h > self.cache.free_pages(g):
-                raise OutOfPagesError(
-                    f"the step needs {h} more pages in cache group {g}, {self.cache.free_pages(g)} are free")
-        for e in entries:
-            self.cache.reserve(e.rid, len(e.tokens))
+    def _reserve(self, entries: Sequence[StepEntry]) -> List[int]:
+        """Pages for the step's new tokens: the whole step or nothing (OutOfPagesError before
+        any page is taken).  Returns the requests' slots."""
+        slots = [self.cache.slot(e.rid) for e in entries]
+        self.cache.reserve_step(slots, [len(e.tokens) for e in entries])
+        return slots
 
     @torch.no_grad()
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
@@ -187,11 +181,10 @@ class ModelRunner:
         if not entries:
             return None
         self._check(entries)
-        self._reserve(entries)
+        slots = self._reserve(entries)
         ctx = self.build_context(entries)
         logits = self.model.forward(ctx, self.layer_caches)
-        for e in entries:
-            self.cache.commit(e.rid, len(e.tokens))
+        self.cache.commit_step(slots, [len(e.tokens) for e in entries])
         return logits
 
     @torch.no_grad()
@@ -204,15 +197,15 @@ class ModelRunner:
         self._check(entries)
         if any(len(e.tokens) != 1 for e in entries):
             raise RequestError("decode_step takes exactly one token per request")
-        self._reserve(entries)
+        slots = self._reserve(entries)
+        lengths = self.cache.lengths_of(slots)
         # one graph per batch size and length bucket: the attention kernel's key ranges follow the bucket
-        bucket = ops.decode_length_bucket(max(self.cache.length(e.rid) for e in entries) + 1)
+        bucket = ops.decode_length_bucket(int(lengths.max()) + 1)
         graph = self._graphs.get((len(entries), bucket))
         if graph is None:
             graph = self._graphs[(len(entries), bucket)] = _DecodeGraph(self, len(entries), bucket)
-        out = graph.run(entries, temperatures, uniforms)
-        for e in entries:
-            self.cache.commit(e.rid, 1)
+        out = graph.run(entries, slots, lengths, temperatures, uniforms)
+        self.cache.commit_step(slots, [1] * len(slots))
         return out
 
 
@@ -273,10 +266,8 @@ class _DecodeGraph:
         self.sampled = torch.zeros(R, dtype=torch.int32, device=runner.device)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
 
-    def _fill(self, entries, temperatures, uniforms) -> None:
+    def _fill(self, entries, slots, lengths, temperatures, uniforms) -> None:
         cache = self.runner.cache
-        slots = [cache.slot(e.rid) for e in entries]
-        lengths = np.fromiter((cache.length(e.rid) for e in entries), np.int32, self.R)
         self.h["token_ids"][:] = [e.tokens[0] for e in entries]
         self.h["positions"][:] = lengths
         self.h["kv_len"][:] = lengths + 1
@@ -292,8 +283,8 @@ class _DecodeGraph:
         logits = self.runner.model.forward(self.ctx, self.runner.layer_caches)
         ops.sample(self.sampled, logits, self.temps, self.uniforms)
 
-    def run(self, entries, temperatures, uniforms) -> torch.Tensor:
-        self._fill(entries, temperatures, uniforms)
+    def run(self, entries, slots, lengths, temperatures, uniforms) -> torch.Tensor:
+        self._fill(entries, slots, lengths, temperatures, uniforms)
         if self.graph is None:
             # the first step of this batch size runs eagerly (and does this step's work); the
             # capture that follows records the same launches without running them

@@ -1,9 +1,10 @@
-"""Builds the HIP kernel libraries for gfx950 with hipcc, in-tree.
+"""Builds the native libraries in-tree: the HIP kernel modules for gfx950 with hipcc, and the
+host-side runtime (plain C++, no device code) with the host compiler.
 
-Sources live in ``photon_infer_amd/csrc``; each *module* is a handful of ``.hip`` files
-linked into ``csrc/_build/libphoton_<module>.so``.  A module is compiled when first
-needed (or when its sources changed since the library was built), one hipcc process per
-file in parallel, with a progress line every few seconds on stderr.
+Sources live in ``photon_infer_amd/csrc``; each *module* is a handful of files linked into
+``csrc/_build/libphoton_<module>.so``.  A module is compiled when first needed (or when its
+sources changed since the library was built), one compiler process per file in parallel,
+with a progress line every few seconds on stderr.
 """
 from __future__ import annotations
 
@@ -27,8 +28,12 @@ CSRC_DIR = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__
 MODULES: Dict[str, List[str]] = {
     "core": ["elementwise.hip", "gemm_general.hip", "attention_general.hip", "sampling.hip"],
     "bf16": ["gemm_mfma.hip", "gemm_skinny.hip", "attention_mfma.hip", "attention_decode.hip"],
+    # host only: cache manager bookkeeping (needs no GPU and no hipcc)
+    "runtime": ["runtime/cache.cpp"],
 }
 HEADERS = ["common.h", "mfma.h", "attention_mfma.h"]
+HOST_MODULES = {"runtime"}
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]
 
 ARCH = "gfx950"
 HIPCC_FLAGS = [
@@ -51,6 +56,15 @@ def _hipcc() -> str:
                                "the kernels cannot be built and there is no fallback")
 
 
+def _host_compiler() -> str:
+    for cand in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"), shutil.which("clang++"),
+                 "/opt/rocm/lib/llvm/bin/clang++"):
+        if cand and (os.path.isfile(cand) or shutil.which(cand)):
+            return cand
+    raise KernelLibraryMissing("no C++ compiler was found (looked at $CXX, g++, c++, clang++); "
+                               "the runtime library cannot be built")
+
+
 def _build_dir() -> str:
     d = os.path.join(CSRC_DIR, "_build")
     try:
@@ -67,8 +81,9 @@ def _build_dir() -> str:
 
 
 def source_hash(module: str) -> str:
-    h = hashlib.sha256(" ".join(HIPCC_FLAGS).encode())
-    for name in MODULES[module] + HEADERS:
+    host = module in HOST_MODULES
+    h = hashlib.sha256(" ".join(HOST_FLAGS if host else HIPCC_FLAGS).encode())
+    for name in MODULES[module] + ([] if host else HEADERS):
         path = os.path.join(CSRC_DIR, name)
         if os.path.isfile(path):
             with open(path, "rb") as f:
@@ -108,7 +123,10 @@ def build_module(module: str, force: bool = False, quiet: bool = False) -> str:
     lib = library_path(module)
     if not force and is_current(module):
         return lib
-    hipcc = _hipcc()
+    host = module in HOST_MODULES
+    hipcc = _host_compiler() if host else _hipcc()
+    compile_flags = HOST_FLAGS if host else HIPCC_FLAGS
+    link_flags = ["-shared", "-fPIC"] if host else [f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc"]
     bdir = _build_dir()
     sources = MODULES[module]
     missing = [s for s in sources if not os.path.isfile(os.path.join(CSRC_DIR, s))]
@@ -116,7 +134,7 @@ def build_module(module: str, force: bool = False, quiet: bool = False) -> str:
         raise KernelLibraryMissing(f"kernel sources missing for module '{module}': {missing}")
     t0 = time.time()
     if not quiet:
-        _log(f"building kernel module '{module}' for {ARCH} ({len(sources)} files) ...")
+        _log(f"building module '{module}' for {'the host' if host else ARCH} ({len(sources)} files) ...")
     done = threading.Event()
 
     def heartbeat():
@@ -129,8 +147,8 @@ def build_module(module: str, force: bool = False, quiet: bool = False) -> str:
     objs = []
     try:
         def compile_one(src: str) -> str:
-            obj = os.path.join(bdir, f"{module}_{os.path.splitext(src)[0]}.{os.getpid()}.o")
-            _run([hipcc, *HIPCC_FLAGS, "-I", CSRC_DIR, "-c", os.path.join(CSRC_DIR, src), "-o", obj], src)
+            obj = os.path.join(bdir, f"{module}_{os.path.splitext(os.path.basename(src))[0]}.{os.getpid()}.o")
+            _run([hipcc, *compile_flags, "-I", CSRC_DIR, "-c", os.path.join(CSRC_DIR, src), "-o", obj], src)
             if not quiet:
                 _log(f"  compiled {src} ({time.time() - t0:.0f} s)")
             return obj
@@ -138,7 +156,7 @@ def build_module(module: str, force: bool = False, quiet: bool = False) -> str:
         with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
             objs = list(pool.map(compile_one, sources))
         tmp = f"{lib}.{os.getpid()}.tmp"
-        _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", tmp], f"libphoton_{module}.so")
+        _run([hipcc, *link_flags, *objs, "-o", tmp], f"libphoton_{module}.so")
         os.replace(tmp, lib)
         with open(lib + ".hash", "w") as f:
             f.write(source_hash(module))

@@ -147,14 +147,16 @@ def test_mixed_requests_with_pages_used_again(model_dirs, tmp_path, name, dtype)
     assert need < sum(-(-n // 64) * 64 for n in lengths)       # the pool cannot hold them all: pages come back
     runner = runner_for(model_dirs[name], name, dtype, need)
     owners = {}                                                # page -> requests that held it
-    orig_reserve = runner.cache.reserve
+    orig_reserve = runner.cache.reserve_step
 
-    def spy(rid, n):
-        orig_reserve(rid, n)
-        for p in runner.cache.table_rows(0, [runner.cache.slot(rid)])[0]:
-            if p >= 0:
-                owners.setdefault(int(p), set()).add(rid)
-    runner.cache.reserve = spy
+    def spy(slots, tokens):
+        orig_reserve(slots, tokens)
+        for rid in list(reqs):
+            if rid in runner.cache and runner.cache.slot(rid) in slots:
+                for p in runner.cache.table_rows(0, [runner.cache.slot(rid)])[0]:
+                    if p >= 0:
+                        owners.setdefault(int(p), set()).add(rid)
+    runner.cache.reserve_step = spy
     got = run_trace(runner, steps, str(tmp_path))
     assert any(len(v) > 1 for v in owners.values()), "no page was handed out a second time"
     check(got, model_dirs[name], reqs, dtype, "mixed")
