@@ -37,6 +37,7 @@ _SIGNATURES = {
     "pi_cache_reserve": (c_int, [c_void_p, c_int, c_int]),
     "pi_cache_commit": (c_int, [c_void_p, c_int, c_int]),
     "pi_cache_release": (c_int, [c_void_p, c_int]),
+    "pi_cache_pages_needed_many": (c_int, [c_void_p, _IP, _IP, c_int, _IP]),
     "pi_cache_reserve_many": (c_int, [c_void_p, _IP, _IP, c_int]),
     "pi_cache_commit_many": (c_int, [c_void_p, _IP, _IP, c_int]),
     "pi_cache_check": (c_int, [c_void_p]),

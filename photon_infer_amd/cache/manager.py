@@ -160,6 +160,16 @@ class CacheManager:
         if status:
             self._fail(status, rid)
 
+    def pages_needed_step(self, rids: Sequence[Hashable], new_tokens: Sequence[int]) -> List[int]:
+        """Pages each group must hand out for all of ``rids`` (live requests) to grow by their
+        ``new_tokens`` in one step."""
+        slots = [self._slots[r] for r in rids]
+        status = self._lib.pi_cache_pages_needed_many(self._h, _native.int_array(slots), _native.int_array(new_tokens),
+                                                      len(slots), self._need)
+        if status:
+            self._fail(status)
+        return list(self._need[:len(self.groups)])
+
     def reserve_step(self, slots: Sequence[int], new_tokens: Sequence[int]) -> None:
         """Pages for a whole step, all or nothing: either every request of the step can grow
         or nothing is taken (OutOfPagesError)."""

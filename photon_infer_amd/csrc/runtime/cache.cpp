@@ -282,6 +282,17 @@ int pi_cache_release(void* h, int slot) {
   return OK;
 }
 
+// Pages each group must hand out for a whole step: every slot growing by its number of tokens.
+int pi_cache_pages_needed_many(void* h, const int* slots, const int* new_tokens, int n, int* out) {
+  Cache* c = static_cast<Cache*>(h);
+  for (size_t g = 0; g < c->groups.size(); ++g) out[g] = 0;
+  for (int i = 0; i < n; ++i) {
+    if (!c->is_live(slots[i])) { c->error = format("slot %d is not live in the cache", slots[i]); return MISUSE; }
+    for (size_t g = 0; g < c->groups.size(); ++g) out[g] += c->needed(c->groups[g], slots[i], new_tokens[i]);
+  }
+  return OK;
+}
+
 // A whole step at once: check that everything fits (nothing is taken otherwise), then reserve.
 int pi_cache_reserve_many(void* h, const int* slots, const int* new_tokens, int n) {
   Cache* c = static_cast<Cache*>(h);

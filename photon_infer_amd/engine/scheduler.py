@@ -245,7 +245,17 @@ class ContinuousBatchScheduler:
 
         # Phase 1: running requests; those with a single token to feed first
         decoding = [r.is_decode() for r in self.running]
-        order = [r for r, d in zip(self.running, decoding) if d] + [r for r, d in zip(self.running, decoding) if not d]
+        order = None
+        if self.running and all(decoding) and budget >= len(self.running):
+            # the common step: everyone decodes; one question for all of them
+            need = self.cache.pages_needed_step([r.request_id for r in self.running], [1] * len(self.running))
+            if self._fits(need, held):
+                held = list(need)
+                batch.items = [(r, 1) for r in self.running]
+                budget -= len(self.running)
+                order = []
+        if order is None:
+            order = [r for r, d in zip(self.running, decoding) if d] + [r for r, d in zip(self.running, decoding) if not d]
         for req in order:
             if req not in self.running:      # preempted while serving an earlier one
                 continue

@@ -118,8 +118,12 @@ class ModelRunner:
             n = len(e.tokens)
             if n == 0:
                 raise RequestError(f"request {e.rid!r} brings no tokens")
-            arr = np.asarray(e.tokens)
-            if arr.dtype.kind not in "iu" or arr.min() < 0 or arr.max() >= vocab:
+            if n <= 8:      # single tokens and short portions: plain comparisons beat an array round trip
+                ok = all(isinstance(t, (int, np.integer)) and 0 <= t < vocab for t in e.tokens)
+            else:
+                arr = np.asarray(e.tokens)
+                ok = arr.dtype.kind in "iu" and arr.min() >= 0 and arr.max() < vocab
+            if not ok:
                 bad = [t for t in e.tokens if not (isinstance(t, (int, np.integer)) and 0 <= int(t) < vocab)]
                 raise RequestError(f"request {e.rid!r}: token id {bad[0]} is outside the vocabulary of {vocab}")
             for w in e.want:
