@@ -17,6 +17,18 @@ from .scheduler import ContinuousBatchScheduler, InferenceRequest, ScheduledBatc
 from .step import ModelRunner, StepEntry
 
 
+class _InFlight:
+    """A decode step that runs on the GPU while the host goes on."""
+
+    def __init__(self, reqs: List[InferenceRequest], ids, host):
+        import torch
+        self.reqs = reqs            # in the order of the step's rows
+        self.ids = ids              # the step's tokens on the device
+        self.host = host            # pinned buffer they are copied to
+        self.done = torch.cuda.Event()
+        self.ended: List[InferenceRequest] = []   # requests in this step that had already ended when it was launched
+
+
 class ContinuousBatchEngine:
     def __init__(self, model_dir: Optional[str], options: Optional[EngineOptions] = None, *,
                  runner: Optional[ModelRunner] = None, **option_fields):
@@ -37,6 +49,8 @@ class ContinuousBatchEngine:
         self.sampler = Sampler(self.runner.device)
         self.eos_token_ids = tuple(self.runner.spec.eos_token_ids)
         self.steps = 0
+        # a decode step that was launched and whose tokens have not been read yet
+        self._in_flight: Optional[_InFlight] = None
 
     @property
     def config(self):
@@ -71,13 +85,80 @@ class ContinuousBatchEngine:
 
     # ------------------------------------------------------------------ running
     def step(self) -> List[InferenceRequest]:
-        """Schedule and run one batch; returns the requests that finished in it."""
+        """Schedule and run one batch; returns the requests known to have finished by the end of
+        the call.  With ``lookahead`` a decode step's tokens are read during the next call: the
+        step after it is launched first, from what is certain without them."""
+        if self._in_flight is not None:
+            return self._step_ahead()
         batch = self.scheduler.schedule_next_batch()
         finished = list(batch.finished)
         if batch.empty():
             return finished
         finished += self.execute_batch_step(batch)
         return finished
+
+    # ---- one step ahead
+    def _launch_decode(self, reqs: List[InferenceRequest], feed=None, pending: int = 0) -> None:
+        """Launch a decode step for ``reqs`` and start the copy of its tokens to the host.
+        ``pending``: tokens of each request that are sampled but not yet known here (0 or 1)."""
+        entries = [StepEntry(r.request_id, r.next_tokens(1) if feed is None else [0], [0]) for r in reqs]
+        temps = [r.params.temperature for r in reqs]
+        draws = [uniform_draw(r.params.seed, r.num_generated() + pending) if r.params.temperature > 0 else 0.0 for r in reqs]
+        ids = self.runner.decode_step(entries, temps, draws, feed)
+        fl = _InFlight(reqs, ids, self._token_buffer(len(reqs)))
+        fl.host.copy_(ids, non_blocking=True)
+        fl.done.record()
+        self._in_flight = fl
+        self.steps += 1
+
+    def _token_buffer(self, n: int):
+        import torch
+        # two pinned buffers per size, used in turn: one is still being read when the next copy starts
+        key = (n, self.steps % 2)
+        buf = self._buffers.get(key) if hasattr(self, "_buffers") else None
+        if buf is None:
+            if not hasattr(self, "_buffers"):
+                self._buffers = {}
+            buf = self._buffers[key] = torch.empty(n, dtype=torch.int32, pin_memory=True)
+        return buf
+
+    def _collect(self, fl: "_InFlight", skip: Sequence[InferenceRequest] = ()) -> List[InferenceRequest]:
+        """Read a launched step's tokens and book them; returns the requests they finished."""
+        fl.done.synchronize()
+        done = []
+        for req, tok in zip(fl.reqs, fl.host.tolist()):
+            if req in skip:            # ended a step earlier; this token was computed for nothing
+                continue
+            req.add_computed_tokens(1)
+            if not req.add_token(tok, self.eos_token_ids, self.runner.max_model_len):
+                done.append(req)
+        return done
+
+    def _step_ahead(self) -> List[InferenceRequest]:
+        fl, self._in_flight = self._in_flight, None
+        sched = self.scheduler
+        # who certainly goes on after the step in flight: everyone it does not end by length.
+        # An end token would end one more, which is only known once the tokens are here.
+        nxt = [r for r in fl.reqs if r not in fl.ended and r.num_generated() + 1 < r.max_new_tokens
+               and r.total_tokens() + 1 <= self.runner.max_model_len]
+        # only when the step in flight is all there is to run (nobody waits, nobody else runs),
+        # the token budget allows it and every next page is there; otherwise the scheduler decides
+        ahead = (bool(nxt) and not sched.waiting and len(sched.running) == len(fl.reqs)
+                 and len(nxt) <= sched.max_step_tokens
+                 and all(n <= self.runner.cache.free_pages(g)
+                         for g, n in enumerate(self.runner.cache.pages_needed_step([r.request_id for r in nxt], [1] * len(nxt)))))
+        if ahead:
+            rows = [fl.reqs.index(r) for r in nxt] if len(nxt) != len(fl.reqs) else list(range(len(nxt)))
+            self._launch_decode(nxt, feed=(fl.ids, rows), pending=1)
+            sched.note_step(len(nxt))
+        done = self._collect(fl, skip=fl.ended)
+        if self._in_flight is not None:
+            # requests that an end token finished are in the step just launched: they leave when it is read
+            self._in_flight.ended = [r for r in done if r in self._in_flight.reqs]
+            sched.update_after_step([r for r in done if r not in self._in_flight.reqs] + list(fl.ended))
+        else:
+            sched.update_after_step(done + list(fl.ended))
+        return done
 
     def execute_batch_step(self, batch: ScheduledBatch) -> List[InferenceRequest]:
         entries, sampled_reqs = [], []
@@ -92,6 +173,9 @@ class ContinuousBatchEngine:
         tokens: List[int] = []
         if self.options.use_graphs and len(sampled_reqs) == len(entries) and all(n == 1 for _, n in batch.items):
             # single tokens only, every one sampled: the replayed graph (model + sampling kernel)
+            if self.options.lookahead:
+                self._launch_decode(sampled_reqs)
+                return []                   # its tokens are read in the next call
             tokens = self.runner.decode_step(entries, temps, draws).tolist()
         else:
             logits = self.runner.step(entries)
@@ -108,7 +192,7 @@ class ContinuousBatchEngine:
         return done
 
     def run_until_complete(self, print_progress: bool = False) -> None:
-        while self.scheduler.has_work():
+        while self.scheduler.has_work() or self._in_flight is not None:
             if print_progress and self.steps % 10 == 0:
                 s = self.scheduler.get_stats()
                 print(f"Step {self.steps}: Running={s.num_running} Waiting={s.num_waiting} Finished={s.num_finished}",

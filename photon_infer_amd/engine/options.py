@@ -41,6 +41,7 @@ class EngineOptions:
     seed: int = 0
     device: str = "cuda:0"
     use_graphs: bool = True              # replay HIP graphs for decode-only steps
+    lookahead: bool = True               # schedule a decode step while the one before it still runs (needs use_graphs)
 
     def resolved_dtype(self) -> torch.dtype:
         return parse_dtype(self.dtype)

@@ -310,6 +310,11 @@ class ContinuousBatchScheduler:
         self._tokens += batch.num_tokens()
         return batch
 
+    def note_step(self, tokens: int) -> None:
+        """A step that was launched without asking (the engine's step ahead) counts too."""
+        self._steps += 1
+        self._tokens += tokens
+
     def update_after_step(self, finished: Sequence[InferenceRequest]) -> None:
         """Requests that ended in this step leave the running list and the cache."""
         for req in finished:

@@ -192,15 +192,25 @@ class ModelRunner:
         return logits
 
     @torch.no_grad()
-    def decode_step(self, entries: Sequence[StepEntry], temperatures: Sequence[float],
-                    uniforms: Sequence[float]) -> torch.Tensor:
+    def decode_step(self, entries: Sequence[StepEntry], temperatures: Sequence[float], uniforms: Sequence[float],
+                    feed: Optional[Tuple[torch.Tensor, Sequence[int]]] = None) -> torch.Tensor:
         """A batch of single tokens, one per request, each wanting its next token: the model
-        and the sampling kernel run as one replayed HIP graph (captured per batch size at
-        first use).  Returns the chosen token ids (int32 [R], on the device)."""
+        and the sampling kernel run as one replayed HIP graph (captured per batch size and
+        length bucket at first use).  Returns the chosen token ids (int32 [R], on the device);
+        the same buffer is written by the next step of the same shape, so read or copy it
+        before launching that one.
+
+        ``feed`` = (ids, rows): the tokens are not known on the host yet; request i's token is
+        ``ids[rows[i]]``, taken on the device (``ids``: what an earlier decode_step returned).
+        The entries' own token values are then ignored."""
         entries = list(entries)
-        self._check(entries)
         if any(len(e.tokens) != 1 for e in entries):
             raise RequestError("decode_step takes exactly one token per request")
+        if feed is not None:
+            if len(feed[1]) != len(entries):
+                raise RequestError("decode_step: one fed row per request is needed")
+            entries = [StepEntry(e.rid, [0], e.want) for e in entries]     # placeholders pass the vocabulary check
+        self._check(entries)
         slots = self._reserve(entries)
         lengths = self.cache.lengths_of(slots)
         # one graph per batch size and length bucket: the attention kernel's key ranges follow the bucket
@@ -208,7 +218,7 @@ class ModelRunner:
         graph = self._graphs.get((len(entries), bucket))
         if graph is None:
             graph = self._graphs[(len(entries), bucket)] = _DecodeGraph(self, len(entries), bucket)
-        out = graph.run(entries, slots, lengths, temperatures, uniforms)
+        out = graph.run(entries, slots, lengths, temperatures, uniforms, feed)
         self.cache.commit_step(slots, [1] * len(slots))
         return out
 
@@ -242,7 +252,7 @@ class _DecodeGraph:
         # no request of this graph is longer than the bucket: its tables need no more columns
         self.width = min(cache.max_blocks, -(-length_bucket // cache.page_size))
         G = len(cache.groups)
-        names = ["token_ids", "positions", "req_of_token", "kv_len", "slots", "logit_rows", "temps", "uniforms"]
+        names = ["token_ids", "positions", "req_of_token", "kv_len", "slots", "logit_rows", "temps", "uniforms", "feed_rows"]
         self.off, total = {}, 0
         for name in names:
             self.off[name] = (total, R)
@@ -252,12 +262,19 @@ class _DecodeGraph:
         for g in range(G):
             self.off[f"table{g}"] = (total, R * self.width)
             total += (R * self.width + 3) // 4 * 4
-        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
-        self.h = {k: self.host[o:o + n].numpy() for k, (o, n) in self.off.items()}
-        self.hf = {k: self.host[o:o + n].view(torch.float32).numpy() for k, (o, n) in self.off.items() if k in ("temps", "uniforms")}
-        self.h["req_of_token"][:] = np.arange(R)
-        self.h["logit_rows"][:] = np.arange(R)
-        self.h["q_start"][:] = np.arange(R + 1)
+        # two pinned staging buffers, used in turn: a step may be filled while the copy of the
+        # one before it has not run yet (the engine launches one step ahead)
+        self._staging = []
+        for _ in range(2):
+            host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+            h = {k: host[o:o + n].numpy() for k, (o, n) in self.off.items()}
+            hf = {k: host[o:o + n].view(torch.float32).numpy() for k, (o, n) in self.off.items() if k in ("temps", "uniforms")}
+            h["req_of_token"][:] = np.arange(R)
+            h["logit_rows"][:] = np.arange(R)
+            h["q_start"][:] = np.arange(R + 1)
+            self._staging.append((host, h, hf))
+        self._turn = 0
+        self.host, self.h, self.hf = self._staging[0]
         self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
         d = {k: self.dev[o:o + n] for k, (o, n) in self.off.items()}
         self.ctx = StepContext(
@@ -265,14 +282,20 @@ class _DecodeGraph:
             req_of_token=d["req_of_token"], q_start=d["q_start"], kv_len=d["kv_len"], slots=d["slots"],
             block_tables={g: d[f"table{g}"].view(R, self.width) for g in range(G)}, logit_rows=d["logit_rows"],
             q_lens=[1] * R, kv_lens=(), max_q_len=1, max_kv_len=length_bucket, all_decode=True)
+        self.feed_rows = d["feed_rows"]
         self.temps = d["temps"].view(torch.float32)
         self.uniforms = d["uniforms"].view(torch.float32)
         self.sampled = torch.zeros(R, dtype=torch.int32, device=runner.device)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
 
-    def _fill(self, entries, slots, lengths, temperatures, uniforms) -> None:
+    def _fill(self, entries, slots, lengths, temperatures, uniforms, feed) -> None:
         cache = self.runner.cache
-        self.h["token_ids"][:] = [e.tokens[0] for e in entries]
+        self._turn ^= 1
+        self.host, self.h, self.hf = self._staging[self._turn]
+        if feed is None:
+            self.h["token_ids"][:] = [e.tokens[0] for e in entries]
+        else:
+            self.h["feed_rows"][:] = feed[1]
         self.h["positions"][:] = lengths
         self.h["kv_len"][:] = lengths + 1
         self.h["slots"][:] = slots
@@ -282,13 +305,15 @@ class _DecodeGraph:
             self.h[f"table{g}"].reshape(self.R, self.width)[:] = cache.table_rows(g, slots, self.width)
         self.ctx.host_slots = slots
         self.dev.copy_(self.host, non_blocking=True)
+        if feed is not None:      # the tokens come from an earlier step's result, on the device
+            torch.index_select(feed[0], 0, self.feed_rows, out=self.ctx.token_ids)
 
     def _body(self) -> None:
         logits = self.runner.model.forward(self.ctx, self.runner.layer_caches)
         ops.sample(self.sampled, logits, self.temps, self.uniforms)
 
-    def run(self, entries, slots, lengths, temperatures, uniforms) -> torch.Tensor:
-        self._fill(entries, slots, lengths, temperatures, uniforms)
+    def run(self, entries, slots, lengths, temperatures, uniforms, feed=None) -> torch.Tensor:
+        self._fill(entries, slots, lengths, temperatures, uniforms, feed)
         if self.graph is None:
             # the first step of this batch size runs eagerly (and does this step's work); the
             # capture that follows records the same launches without running them

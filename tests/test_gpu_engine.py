@@ -164,3 +164,56 @@ def test_graph_replayed_decode_equals_eager_steps(tmp_path, dtype, name):
     assert all(g.graph is not None for g in eng.runner._graphs.values())
     assert graphed == eager
     assert [len(x) for x in graphed] == [14, 17, 20, 9]
+
+
+@pytest.mark.parametrize("dtype,name", [("float32", "A"), ("bfloat16", "D")])
+def test_a_step_ahead_gives_the_same_tokens(tmp_path, dtype, name):
+    """Launching the next decode step before this one's tokens are on the host (they are fed
+    back on the device) changes nothing: requests of different lengths ending at different
+    steps, greedy and sampled, one arriving mid-run."""
+    d = make_model_dir(tmp_path, name, seed=33)
+    vocab = ALL[name][0]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 70 + n) for n in (4, 21, 9, 15)]
+
+    def run(lookahead):
+        eng = engine(d, name, dtype=dtype, lookahead=lookahead, chunk_size=8, max_step_tokens=32)
+        ids = [eng.add_request(p, 5 + 6 * i, temperature=0.9 if i % 2 else 0.0, seed=3 + i, ignore_eos=True)
+               for i, p in enumerate(prompts[:3])]
+        for _ in range(9):
+            eng.step()
+        ids.append(eng.add_request(prompts[3], 11, temperature=0.5, seed=9, ignore_eos=True))
+        eng.run_until_complete()
+        assert eng.runner.cache.num_live == 0 and eng.get_stats().num_finished == 4
+        eng.runner.cache.check_invariants()
+        return [eng.get_result(i) for i in ids]
+
+    plain, ahead = run(False), run(True)
+    assert ahead == plain
+    assert [len(x) for x in ahead] == [5, 11, 17, 11]
+
+
+def test_an_end_token_during_a_step_ahead(tmp_path):
+    """An end token is only seen one step late: the request's row in the step already launched
+    is wasted, its result must not be, and its pages go back when that step has been read."""
+    d = make_model_dir(tmp_path, "A", seed=35)
+    prompts = [random_tokens(n, 256, 80 + n) for n in (6, 13, 3)]
+    free = engine(d, "A", lookahead=False).generate(prompts, max_new_tokens=12, ignore_eos=True)
+    # an end token that the second request produces mid-way and that cuts it short
+    stop = free[1][5]
+    cut = free[1].index(stop) + 1
+
+    def run(lookahead):
+        eng = engine(d, "A", lookahead=lookahead)
+        eng.eos_token_ids = (stop,)
+        ids = [eng.add_request(p, 12) for p in prompts]
+        eng.run_until_complete()
+        assert eng.runner.cache.num_live == 0 and eng.runner.cache.free_pages() == 128
+        eng.runner.cache.check_invariants()
+        return [eng.get_result(i) for i in ids], [eng.get_request(i).finish_reason for i in ids]
+
+    (plain, why_plain), (ahead, why_ahead) = run(False), run(True)
+    assert ahead == plain and why_ahead == why_plain
+    assert ahead[1] == free[1][:cut] and why_ahead[1] == "eos"
+    for i in (0, 2):                       # the others run on unless they meet the token themselves
+        n = free[i].index(stop) + 1 if stop in free[i] else 12
+        assert ahead[i] == free[i][:n]
