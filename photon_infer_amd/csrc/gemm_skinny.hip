@@ -13,12 +13,16 @@
 // Epilogues as in the many-row kernel: store bf16, store f32, add into f32, SwiGLU (gate / up
 // rows interleaved by 16, so the two row tiles of a wave are the gate and the up rows of the
 // same 16 features; no k-split over blocks in that case).
+#include <type_traits>
+
 #include "mfma.h"
 
 enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACCUM = 2, EPI_SWIGLU = 3 };
 
 #define ROWS_PER_BLOCK 32
 #define KSTEP 64
+#define SHARED_FROM_TOKENS 32   // more tokens than this: the kernel that shares an activation tile per block
+#define SHARED_DEPTH 4          // k steps of loads a wave keeps in flight (measured: more is slower)
 
 template <int EPI>
 __device__ inline void epilogue_store(void* Cv, long ldc, long m, long n, float v) {
@@ -27,11 +31,22 @@ __device__ inline void epilogue_store(void* Cv, long ldc, long m, long n, float 
   if (EPI == EPI_ACCUM) reinterpret_cast<float*>(Cv)[m * ldc + n] += v;
 }
 
+// LDS of a block: while the k loop runs, each wave stages its activations there (the loads from
+// memory follow the rows, eight lanes on a row's 128 bytes, which the cache serves at twice the
+// rate of the operand's own pattern of sixteen rows per quarter wave); afterwards the same bytes
+// hold the waves' partial tiles for the sum.
+template <int MB>
+union SkinnyLds {
+  float red[4][ROWS_PER_BLOCK][MB * 16 + 1];
+  u32x4_t xs[4][MB * 8 * 16];          // per wave: [token tile][16-byte piece of the k step][token], tokens turned by the piece
+};
+
 template <int MB, int EPI>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ X, long ldx,
                                                           const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
                                                           int k_per_block, float* __restrict__ part) {
-  __shared__ float red[4][ROWS_PER_BLOCK][MB * 16 + 1];
+  __shared__ SkinnyLds<MB> lds;
+  float (*red)[ROWS_PER_BLOCK][MB * 16 + 1] = lds.red;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int lr = lane % 16, lg = lane / 16;
   const long n0 = (long)blockIdx.x * ROWS_PER_BLOCK;
@@ -44,13 +59,30 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
   const int k0 = kb0 + wave * per_wave;
   const int k1 = min(kb1, k0 + per_wave);
 
-  // rows beyond N / tokens beyond M read the last valid row; their results are never stored
+  // rows beyond N read the last valid row; their results are never stored
   const bf16_t* wrow[2];
 #pragma unroll
   for (int t = 0; t < 2; ++t) wrow[t] = W + min(n0 + t * 16 + lr, (long)N - 1) * ldw + lg * 16;
-  const bf16_t* xrow[MB];
+
+  // Activations of a k step: load instruction i brings tokens 8i .. 8i+7, lane j the 16-byte
+  // piece j % 8 of token 8i + j / 8.  Tokens beyond M are not loaded: what LDS holds for them
+  // only reaches columns of the result that are never stored.
+  const int x_loads = __builtin_amdgcn_readfirstlane((M + 7) / 8);
+  const int xt = lane / 8, xp = lane % 8;
+  const bf16_t* xsrc[MB * 2];
+  int xdst[MB * 2];
 #pragma unroll
-  for (int c = 0; c < MB; ++c) xrow[c] = X + (long)min(c * 16 + lr, M - 1) * ldx + lg * 16;
+  for (int i = 0; i < MB * 2; ++i) {
+    const int token = i * 8 + xt;
+    xsrc[i] = X + (long)min(token, M - 1) * ldx + xp * 8;
+    xdst[i] = ((token / 16) * 8 + xp) * 16 + ((token + 2 * xp) & 15);
+  }
+  u32x4_t* xs = lds.xs[wave];
+  int xfrag[MB][2];                     // where this lane's operand pieces lie: piece lg*2+h of token lr
+#pragma unroll
+  for (int c = 0; c < MB; ++c)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) xfrag[c][h] = (c * 8 + lg * 2 + h) * 16 + ((lr + 2 * (lg * 2 + h)) & 15);
 
   f32x4_t acc[2][MB];
 #pragma unroll
@@ -58,19 +90,37 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
 #pragma unroll
     for (int c = 0; c < MB; ++c) acc[t][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
-  int kk = k0;
-  for (; kk + KSTEP <= k1; kk += KSTEP) {
-    Frag w[2][2], x[MB][2];
+  // one k step; in a last, partial one the 8-element pieces beyond k1 count as zero
+  auto step = [&](const int kk, auto whole_step) {
+    constexpr bool whole = decltype(whole_step)::value;
+    Frag w[2][2];
+    u32x4_t xg[MB * 2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t) {
-      w[t][0] = load_frag(wrow[t] + kk);
-      w[t][1] = load_frag(wrow[t] + kk + 8);
-    }
+    for (int t = 0; t < 2; ++t)
 #pragma unroll
-    for (int c = 0; c < MB; ++c) {
-      x[c][0] = load_frag(xrow[c] + kk);
-      x[c][1] = load_frag(xrow[c] + kk + 8);
-    }
+      for (int h = 0; h < 2; ++h) {
+        w[t][h] = load_frag(wrow[t] + (whole || kk + lg * 16 + h * 8 < k1 ? kk + h * 8 : k0));
+        if (!whole && kk + lg * 16 + h * 8 >= k1) w[t][h] = zero_frag();
+      }
+    const bool x_ok = whole || kk + xp * 8 < k1;
+#pragma unroll
+    for (int i = 0; i < MB * 2; ++i)
+      if (i == 0 || i < x_loads) {
+        xg[i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + (x_ok ? kk : k0));
+        if (!x_ok) xg[i] = u32x4_t{0u, 0u, 0u, 0u};
+      }
+#pragma unroll
+    for (int i = 0; i < MB * 2; ++i)
+      if (i == 0 || i < x_loads) xs[xdst[i]] = xg[i];
+    // the wave reads what its own lanes wrote: LDS serves one wave's accesses in order
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    Frag x[MB][2];
+#pragma unroll
+    for (int c = 0; c < MB; ++c)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) x[c][h].n = xs[xfrag[c][h]];
 #pragma unroll
     for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -78,23 +128,13 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
         acc[t][c] = mfma16(w[t][0], x[c][0], acc[t][c]);
         acc[t][c] = mfma16(w[t][1], x[c][1], acc[t][c]);
       }
-  }
-  if (kk < k1) {  // a last, partial step: 8-element chunks beyond k1 count as zero
-    const int ka = kk + lg * 16;
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const bool ok = ka + h * 8 < k1;
-      Frag w[2], x[MB];
-#pragma unroll
-      for (int t = 0; t < 2; ++t) w[t] = ok ? load_frag(wrow[t] + kk + h * 8) : zero_frag();
-#pragma unroll
-      for (int c = 0; c < MB; ++c) x[c] = ok ? load_frag(xrow[c] + kk + h * 8) : zero_frag();
-#pragma unroll
-      for (int t = 0; t < 2; ++t)
-#pragma unroll
-        for (int c = 0; c < MB; ++c) acc[t][c] = mfma16(w[t], x[c], acc[t][c]);
-    }
-  }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+  };
+  int kk = k0;
+  for (; kk + KSTEP <= k1; kk += KSTEP) step(kk, std::true_type{});
+  if (kk < k1) step(kk, std::false_type{});
+  __syncthreads();                      // the partial tiles take the place of the staged activations
 
   // acc[t][c][r] is C^T[n0 + t*16 + lg*4 + r][c*16 + lr]; add the four waves through LDS
 #pragma unroll
@@ -138,6 +178,138 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
   }
 }
 
+// The same product for 33..64 tokens, where the activations are as many bytes as a block's
+// weights: the four waves of a block take 16 weight rows each over the block's whole k-range
+// and share one activation tile per k step through LDS (loaded once per block, not once per
+// wave).  A block is alone on its compute unit, so every wave keeps DEPTH k steps of loads
+// (weights and its share of the activation tile) in flight in registers; loads return in
+// order, which is why both travel at the same distance.
+#define SHARED_ROWS_PER_BLOCK 64
+
+template <int MB, int EPI, int DEPTH>
+__global__ __launch_bounds__(256) void gemm_skinny_shared_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ X, long ldx,
+                                                                 const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
+                                                                 int k_per_block, float* __restrict__ part) {
+  constexpr int ROWS = SHARED_ROWS_PER_BLOCK;
+  constexpr int XL = (MB + 1) / 2;      // 16-byte pieces of an activation tile per lane
+  __shared__ union {
+    u32x4_t xs[2][MB * 128];            // [token tile][piece of the k step][token], tokens turned by the piece
+    float tile[ROWS][MB * 16 + 1];
+  } lds;
+  const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+  const int lr = lane % 16, lg = lane / 16;
+  const long n0 = (long)blockIdx.x * ROWS;
+  const int splits = gridDim.y;
+  const int kb0 = blockIdx.y * k_per_block;
+  const int kb1 = min(K, kb0 + k_per_block);
+  const int steps = (kb1 - kb0 + KSTEP - 1) / KSTEP;
+  auto k_of = [&](const int s) { return kb0 + min(s, steps - 1) * KSTEP; };   // steps beyond the last are fetched, never used
+
+  // rows beyond N and tokens beyond M read the last valid one; their results are never stored
+  const bf16_t* wrow = W + min(n0 + wave * 16 + lr, (long)N - 1) * ldw;
+  const int xp = tid % 8;
+  const bf16_t* xsrc[XL];
+  int xdst[XL];
+  bool xmine[XL];
+#pragma unroll
+  for (int i = 0; i < XL; ++i) {
+    const int token = i * 32 + tid / 8;
+    xsrc[i] = X + (long)min(token, M - 1) * ldx;
+    xdst[i] = ((token / 16) * 8 + xp) * 16 + ((token + 2 * xp) & 15);
+    xmine[i] = token < MB * 16;
+  }
+  int xfrag[MB][2];
+#pragma unroll
+  for (int c = 0; c < MB; ++c)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) xfrag[c][h] = (c * 8 + lg * 2 + h) * 16 + ((lr + 2 * (lg * 2 + h)) & 15);
+
+  f32x4_t acc[MB];
+#pragma unroll
+  for (int c = 0; c < MB; ++c) acc[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+
+  Frag wq[DEPTH][2];
+  u32x4_t xq[DEPTH][XL];
+  // every step issues the same loads, also beyond the range (clamped, never used): the count
+  // of loads in flight is then a constant the compiler can wait on exactly
+  auto fetch = [&](const int s, const int j) {
+    const int kk = k_of(s);
+#pragma unroll
+    for (int i = 0; i < XL; ++i) xq[j][i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + min(kk + xp * 8, kb1 - 8));
+#pragma unroll
+    for (int h = 0; h < 2; ++h) wq[j][h] = load_frag(wrow + min(kk + lg * 16 + h * 8, kb1 - 8));
+  };
+#pragma unroll
+  for (int j = 0; j < DEPTH; ++j) fetch(j, j);
+
+  // the tile of step s + 1 goes to LDS (the other of two buffers) before step s computes, so
+  // that the one barrier per step finds every wave's writes long done
+  auto stage = [&](const int s, const int j) {
+    const bool x_ok = k_of(s) + xp * 8 < kb1;          // 8-element pieces beyond the range count as zero
+    u32x4_t* xs = lds.xs[s & 1];
+#pragma unroll
+    for (int i = 0; i < XL; ++i)
+      if (xmine[i]) xs[xdst[i]] = x_ok ? xq[j][i] : u32x4_t{0u, 0u, 0u, 0u};
+  };
+  auto step = [&](const int s, const int j, auto more_to_fetch) {
+    const int kk = k_of(s);
+    stage(s + 1, (j + 1) % DEPTH);
+    const u32x4_t* xs = lds.xs[s & 1];
+    Frag x[MB][2], w[2];
+#pragma unroll
+    for (int c = 0; c < MB; ++c)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) x[c][h].n = xs[xfrag[c][h]];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) w[h].n = kk + lg * 16 + h * 8 < kb1 ? wq[j][h].n : u32x4_t{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int c = 0; c < MB; ++c) acc[c] = mfma16(w[h], x[c][h], acc[c]);
+    if (decltype(more_to_fetch)::value) fetch(s + DEPTH, j);
+    __syncthreads();
+  };
+  stage(0, 0);
+  __syncthreads();
+  // whole rounds of DEPTH steps have no branch, so that the waits stay exact; the last steps
+  // fetch nothing more
+  int s0 = 0;
+  for (; s0 + DEPTH <= steps; s0 += DEPTH) {
+#pragma unroll
+    for (int j = 0; j < DEPTH; ++j) step(s0 + j, j, std::true_type{});
+  }
+#pragma unroll
+  for (int j = 0; j < DEPTH; ++j)
+    if (s0 + j < steps) step(s0 + j, j, std::false_type{});
+  // (the last step ended with a barrier: the result tile may take the place of the activation tiles)
+
+  // acc[c][r] is C^T[n0 + wave*16 + lg*4 + r][c*16 + lr]
+#pragma unroll
+  for (int c = 0; c < MB; ++c)
+#pragma unroll
+    for (int r = 0; r < 4; ++r) lds.tile[wave * 16 + lg * 4 + r][c * 16 + lr] = acc[c][r];
+  __syncthreads();
+
+  const int cols = MB * 16;
+  if (splits == 1 && EPI == EPI_SWIGLU) {
+    // rows [gate 16 | up 16 | gate 16 | up 16]: 32 features per block
+    for (int idx = tid; idx < 32 * cols; idx += 256) {
+      const int j = idx % 16, pair = (idx / 16) % 2, m = idx / 32;
+      if (m >= M || n0 + pair * 32 + 16 + j >= N) continue;
+      const float g = lds.tile[pair * 32 + j][m], u = lds.tile[pair * 32 + 16 + j][m];
+      reinterpret_cast<bf16_t*>(Cv)[(long)m * ldc + n0 / 2 + pair * 16 + j] = from_float<bf16_t>(g / (1.0f + expf(-g)) * u);
+    }
+    return;
+  }
+  float* mine = part + (long)blockIdx.y * M * N;
+  for (int idx = tid; idx < ROWS * cols; idx += 256) {
+    const int nl = idx % ROWS, m = idx / ROWS;
+    if (m >= M || n0 + nl >= N) continue;
+    if (splits == 1) epilogue_store<EPI>(Cv, ldc, m, n0 + nl, lds.tile[nl][m]);
+    else mine[(long)m * N + n0 + nl] = lds.tile[nl][m];   // the consumer adds the splits in split order
+  }
+}
+
 // C[m][n] (op)= sum over splits of part[s][m][n], in split order.
 template <int EPI>
 __global__ void splitk_reduce_kernel(void* __restrict__ Cv, long ldc, const float* __restrict__ part, int splits, int M, int N) {
@@ -177,6 +349,24 @@ static int launch_mb(int epi, dim3 grid, hipStream_t stream, void* C, long ldc, 
   return pi_check_launch("gemm_skinny");
 }
 
+template <int MB>
+static int launch_shared(int epi, dim3 grid, hipStream_t stream, void* C, long ldc, const bf16_t* X, long ldx, const bf16_t* W,
+                         long ldw, int M, int N, int K, int kpb, float* part) {
+#define GO(E) hipLaunchKernelGGL((gemm_skinny_shared_kernel<MB, E, SHARED_DEPTH>), grid, dim3(256), 0, stream, C, ldc, X, ldx, W, ldw, M, N, K, kpb, part)
+  switch (epi) {
+    case EPI_BF16: GO(EPI_BF16); break;
+    case EPI_F32: GO(EPI_F32); break;
+    case EPI_ACCUM: GO(EPI_ACCUM); break;
+    case EPI_SWIGLU: GO(EPI_SWIGLU); break;
+    default: return pi_fail("gemm_skinny: unknown epilogue %d", epi);
+  }
+#undef GO
+  return pi_check_launch("gemm_skinny (shared activations)");
+}
+
+// Rows of the weight matrix per block for M tokens (the caller sizes its k-split by it).
+extern "C" int pi_gemm_skinny_rows_per_block(int M) { return M > SHARED_FROM_TOKENS ? SHARED_ROWS_PER_BLOCK : ROWS_PER_BLOCK; }
+
 // splits > 1: the partial products go to `part` (float32 [splits, M, N]) and C is not touched;
 // *splits_out tells how many splits were made (no empty ones).
 extern "C" int pi_gemm_skinny(void* C, int epilogue, long ldc, const void* X, long ldx, const void* W, long ldw, int M,
@@ -186,7 +376,7 @@ extern "C" int pi_gemm_skinny(void* C, int epilogue, long ldc, const void* X, lo
   PI_REQUIRE(((uintptr_t)X % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_skinny: operands must be 16-byte aligned");
   PI_REQUIRE(splits >= 1 && splits <= 65535, "gemm_skinny: bad split count %d", splits);
   PI_REQUIRE(epilogue != EPI_SWIGLU || (splits == 1 && N % 32 == 0), "gemm_skinny: the SwiGLU epilogue needs one split and N (%d) a multiple of 32", N);
-  const int groups = ceil_div(N, ROWS_PER_BLOCK);
+  const int groups = ceil_div(N, pi_gemm_skinny_rows_per_block(M));
   int kpb = ceil_div(K, splits);
   kpb = ((kpb + KSTEP - 1) / KSTEP) * KSTEP;
   splits = ceil_div(K, kpb);                      // no empty splits
@@ -196,6 +386,9 @@ extern "C" int pi_gemm_skinny(void* C, int epilogue, long ldc, const void* X, lo
   const dim3 grid(groups, splits);
   const int mb = (M + 15) / 16;
   const bf16_t *x = (const bf16_t*)X, *w = (const bf16_t*)W;
+  if (M > SHARED_FROM_TOKENS)
+    return mb == 3 ? launch_shared<3>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part)
+                   : launch_shared<4>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
   switch (mb) {
     case 1: return launch_mb<1>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
     case 2: return launch_mb<2>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);

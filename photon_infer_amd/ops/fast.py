@@ -26,6 +26,9 @@ EPI_BF16, EPI_F32, EPI_ACCUM, EPI_SWIGLU = 0, 1, 2, 3
 SKINNY_MAX_ROWS = 64
 ROWS_PER_BLOCK = 32            # weight rows per block of the skinny kernel
 TARGET_BLOCKS = 512            # blocks wanted in flight to keep HBM busy
+SHARED_FROM_TOKENS = 32        # more tokens than this: the skinny kernel that shares activations per block ...
+SHARED_ROWS_PER_BLOCK = 64     # ... with this many weight rows per block ...
+SHARED_TARGET_BLOCKS = 256     # ... and this many blocks wanted (one per compute unit)
 GEMM_PART_FLOATS = 16 << 20    # workspace for the pieces of products split over k (64 MB)
 TILE_MAX_SPLITS = 4
 ATTN_PART_FLOATS = 4 << 20     # key-split partial results of decode attention
@@ -79,8 +82,11 @@ def _gemm_ok(a, w, K, lda, ldw) -> bool:
 
 
 def _skinny_splits(M: int, N: int, K: int) -> int:
-    groups = -(-N // ROWS_PER_BLOCK)
-    splits = max(1, min(-(-TARGET_BLOCKS // groups), K // 256))
+    if M > SHARED_FROM_TOKENS:     # the kernel that shares an activation tile per block: one block per compute unit
+        groups, wanted = -(-N // SHARED_ROWS_PER_BLOCK), SHARED_TARGET_BLOCKS
+    else:
+        groups, wanted = -(-N // ROWS_PER_BLOCK), TARGET_BLOCKS
+    splits = max(1, min(-(-wanted // groups), K // 256))
     while splits > 1 and splits * M * N > GEMM_PART_FLOATS:
         splits -= 1
     return splits
