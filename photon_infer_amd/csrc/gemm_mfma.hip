@@ -12,6 +12,8 @@
 // Any M and N (edges read zeros and are skipped on store); K must be a multiple of
 // 8 and row strides multiples of 8 so that 16-byte loads stay aligned.  Each output row
 // accumulates over k in the same order whatever the other rows are.
+#include <type_traits>
+
 #include "mfma.h"
 
 PI_DEFINE_MODULE(bf16)
@@ -28,6 +30,93 @@ enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACCUM = 2, EPI_SWIGLU = 3 };
 // far inside the rounding of the store
 __device__ inline float silu_mul(float g, float u) {
   return g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g)) * u;
+}
+
+// The epilogue of both kernels: 32 rows x 64 columns of a wave's result, held as two 32 x 32
+// accumulator tiles (lane = column, register = row), go through a patch of LDS that belongs to
+// the wave alone and come back with eight (bfloat16) or four (float32) neighbouring columns in
+// one lane, so that a row leaves as whole 16-byte stores instead of 2- or 4-byte ones.
+// `C` points at the corner's first element (for SwiGLU: of the halved output); rows_left and
+// cols_left (input columns) may be <= 0 or ragged; `wide` says that 16-byte stores are aligned.
+#define PATCH_LD 72                      // floats per patch row: rows r and r + 4 fall on different bank halves
+#define PATCH_FLOATS (32 * PATCH_LD)
+
+__device__ inline uint32_t pack2(float a, float b) { return f32x2_to_bf16x2_bits(a, b); }
+
+template <int EPI>
+__device__ inline void store_rows32(float* patch, const f32x16_t& acc0, const f32x16_t& acc1, void* C, int ld, int row0,
+                                    int rows_left, int cols_left, int lane, bool wide) {
+  const int half = lane / 32, ccol = lane % 32;
+#pragma unroll
+  for (int v = 0; v < 16; ++v) {
+    const int r = 8 * (v / 4) + 4 * half + v % 4;
+    patch[r * PATCH_LD + ccol] = acc0[v];
+    patch[r * PATCH_LD + 32 + ccol] = acc1[v];
+  }
+  // the wave reads what its own lanes wrote: LDS serves one wave's accesses in order
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+  if (EPI == EPI_SWIGLU) {
+    // columns 0..15 of a tile are gate rows of W, 16..31 the up rows of the same features
+    bf16_t* out = reinterpret_cast<bf16_t*>(C);
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+      const int id = pass * 64 + lane, r = id / 4, j = (id % 4) / 2, q = id % 2;
+      const float* g = patch + r * PATCH_LD + j * 32 + q * 8;
+      const int oc = j * 16 + q * 8;                       // output column; its up column in the input is j*32 + 16 + q*8 (+7)
+      if (row0 + r >= rows_left || j * 32 + 16 + q * 8 >= cols_left) continue;
+      const f32x4_t g0 = *reinterpret_cast<const f32x4_t*>(g), g1 = *reinterpret_cast<const f32x4_t*>(g + 4);
+      const f32x4_t u0 = *reinterpret_cast<const f32x4_t*>(g + 16), u1 = *reinterpret_cast<const f32x4_t*>(g + 20);
+      float o[8];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { o[e] = silu_mul(g0[e], u0[e]); o[4 + e] = silu_mul(g1[e], u1[e]); }
+      bf16_t* dst = out + (row0 + r) * ld + oc;
+      if (wide && j * 32 + 16 + q * 8 + 8 <= cols_left) {
+        *reinterpret_cast<u32x4_t*>(dst) = u32x4_t{pack2(o[0], o[1]), pack2(o[2], o[3]), pack2(o[4], o[5]), pack2(o[6], o[7])};
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (j * 32 + 16 + q * 8 + e < cols_left) dst[e] = from_float<bf16_t>(o[e]);
+      }
+    }
+  } else if (EPI == EPI_BF16) {
+    bf16_t* out = reinterpret_cast<bf16_t*>(C);
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+      const int id = pass * 64 + lane, r = id / 8, c = (id % 8) * 8;
+      if (row0 + r >= rows_left || c >= cols_left) continue;
+      const float* src = patch + r * PATCH_LD + c;
+      const f32x4_t a = *reinterpret_cast<const f32x4_t*>(src), b = *reinterpret_cast<const f32x4_t*>(src + 4);
+      bf16_t* dst = out + (row0 + r) * ld + c;
+      if (wide && c + 8 <= cols_left) {
+        *reinterpret_cast<u32x4_t*>(dst) = u32x4_t{pack2(a[0], a[1]), pack2(a[2], a[3]), pack2(b[0], b[1]), pack2(b[2], b[3])};
+      } else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+          if (c + e < cols_left) dst[e] = from_float<bf16_t>(e < 4 ? a[e] : b[e - 4]);
+      }
+    }
+  } else {
+    float* out = reinterpret_cast<float*>(C);
+#pragma unroll
+    for (int pass = 0; pass < 8; ++pass) {
+      const int id = pass * 64 + lane, r = id / 16, c = (id % 16) * 4;
+      if (row0 + r >= rows_left || c >= cols_left) continue;
+      f32x4_t a = *reinterpret_cast<const f32x4_t*>(patch + r * PATCH_LD + c);
+      float* dst = out + (row0 + r) * ld + c;
+      if (wide && c + 4 <= cols_left) {
+        if (EPI == EPI_ACCUM) a += *reinterpret_cast<const f32x4_t*>(dst);
+        *reinterpret_cast<f32x4_t*>(dst) = a;
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (c + e < cols_left) dst[e] = EPI == EPI_ACCUM ? dst[e] + a[e] : a[e];
+      }
+    }
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
 }
 
 // Global loads go through buffer descriptors: a scalar base (the block's first row at its first
@@ -149,35 +238,19 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
     __syncthreads();
   }
 
-  // acc[i][j][v] is C[m0 + wm*64 + i*32 + 8*(v/4) + 4*(lane/32) + v%4][n0 + wn*64 + j*32 + lane%32]
-  const int half = lane / 32, ccol = lane % 32;
+  // acc[i][j][v] is C[m0 + wm*64 + i*32 + 8*(v/4) + 4*(lane/32) + v%4][n0 + wn*64 + j*32 + lane%32].
+  // The loop ended with a barrier, so LDS is free for the waves' patches.  Offsets inside the
+  // wave's corner are 32-bit (the host checks that 128 * ldc fits).
+  {
+    const long mw = m0 + wm * 64, nw = n0 + wn * 64;
+    const int rows_left = (int)min((long)64, M - mw), cols_left = (int)min((long)64, N - nw);   // may be <= 0
+    float* patch = reinterpret_cast<float*>(lds) + wave * PATCH_FLOATS;
+    const int esize = EPI == EPI_BF16 || EPI == EPI_SWIGLU ? 2 : 4;
+    char* corner = reinterpret_cast<char*>(Cv) + (mw * ldc + (EPI == EPI_SWIGLU ? nw / 2 : nw)) * esize;
+    const bool wide = (ldc * esize) % 16 == 0 && reinterpret_cast<uintptr_t>(corner) % 16 == 0;
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
-      const long nb = n0 + wn * 64 + j * 32;
-#pragma unroll
-      for (int v = 0; v < 16; ++v) {
-        const long m = m0 + wm * 64 + i * 32 + 8 * (v / 4) + 4 * half + v % 4;
-        if (EPI == EPI_SWIGLU) {
-          // columns 0..15 of a tile are gate rows of W, 16..31 the up rows of the same features:
-          // the swap leaves the gate value in both 16-lane rows of one result and the up value
-          // in both rows of the other; the lower rows store
-#if defined(__HIP_DEVICE_COMPILE__)
-          const unsigned bits = __float_as_uint(acc[i][j][v]);
-          auto gu = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
-          if (ccol < 16 && m < M && nb + ccol + 16 < N)
-            reinterpret_cast<bf16_t*>(Cv)[m * ldc + nb / 2 + ccol] = from_float<bf16_t>(silu_mul(__uint_as_float(gu[0]), __uint_as_float(gu[1])));
-#endif
-        } else {
-          const long n = nb + ccol;
-          if (m >= M || n >= N) continue;
-          if (EPI == EPI_BF16) reinterpret_cast<bf16_t*>(Cv)[m * ldc + n] = from_float<bf16_t>(acc[i][j][v]);
-          if (EPI == EPI_F32) reinterpret_cast<float*>(Cv)[m * ldc + n] = acc[i][j][v];
-          if (EPI == EPI_ACCUM) reinterpret_cast<float*>(Cv)[m * ldc + n] += acc[i][j][v];
-        }
-      }
-    }
+    for (int i = 0; i < 2; ++i) store_rows32<EPI>(patch, acc[i][0], acc[i][1], corner, (int)ldc, i * 32, rows_left, cols_left, lane, wide);
+  }
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -202,7 +275,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
 #define PI_SCHED_DS_WRITE 0x200
 
 template <int EPI>
-__global__ __launch_bounds__(256) void gemm_mfma_big_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ A, long lda,
+__global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ A, long lda,
                                                             const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
                                                             int tiles_n, int k_per_split) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
@@ -210,7 +283,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_big_kernel(void* __restrict__ C
   uint16_t* Ws = lds + 2 * BIG_TILE_ELEMS;      // [2][GN][LDS_ROW]
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
-  const int wm = wave / 2, wn = wave % 2;
+  const int wm = wave / 4, wn = wave % 4;       // a wave's corner: 128 rows x 64 columns
   const int k_lo = blockIdx.y * k_per_split;
   const int k_hi = min(K, k_lo + k_per_split);
   if (gridDim.y > 1) Cv = reinterpret_cast<float*>(Cv) + (long)blockIdx.y * M * ldc;
@@ -226,7 +299,7 @@ __global__ __launch_bounds__(256) void gemm_mfma_big_kernel(void* __restrict__ C
   }
   const long m0 = (long)tile_m * GM, n0 = (long)tile_n * GN;
 
-  // global -> registers: thread t moves 16-byte chunk t % 8 of rows lrow + 32 p of both operands
+  // global -> registers: thread t moves 16-byte chunk t % 8 of rows lrow + 64 p of both operands
   const int lgrp = tid / 8, lchunk = tid % 8;
   const int lrow = (lgrp / 16) * 16 + ((lgrp / 8) % 2) * 4 + (lgrp % 8) / 2 + 8 * (lgrp % 2);
   const int a_rows = (int)min((long)GM, M - m0), w_rows = (int)min((long)GN, N - n0);
@@ -234,19 +307,19 @@ __global__ __launch_bounds__(256) void gemm_mfma_big_kernel(void* __restrict__ C
   const __amdgpu_buffer_rsrc_t a_src = operand_descriptor(A + m0 * lda + k_lo, ((long)(a_rows - 1) * lda + (k_hi - k_lo)) * 2);
   const __amdgpu_buffer_rsrc_t w_src = operand_descriptor(W + n0 * ldw + k_lo, ((long)(w_rows - 1) * ldw + (k_hi - k_lo)) * 2);
 #endif
-  unsigned a_off[8], w_off[8];
+  unsigned a_off[4], w_off[4];
 #pragma unroll
-  for (int p = 0; p < 8; ++p) {
-    a_off[p] = (unsigned)(min(lrow + 32 * p, a_rows - 1) * (int)lda + lchunk * 8) * 2u;
-    w_off[p] = (unsigned)(min(lrow + 32 * p, w_rows - 1) * (int)ldw + lchunk * 8) * 2u;
+  for (int p = 0; p < 4; ++p) {
+    a_off[p] = (unsigned)(min(lrow + 64 * p, a_rows - 1) * (int)lda + lchunk * 8) * 2u;
+    w_off[p] = (unsigned)(min(lrow + 64 * p, w_rows - 1) * (int)ldw + lchunk * 8) * 2u;
   }
-  u32x4_t ra[8], rw[8];
+  u32x4_t ra[4], rw[4];
   const int slabs = (k_hi - k_lo) / BK;
   auto load_slab = [&](int s) {
     const int kbytes = min(s, slabs - 1) * BK * 2;     // past the last slab: read it again, unused
 #if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
+    for (int p = 0; p < 4; ++p) {
       ra[p] = __builtin_amdgcn_raw_buffer_load_b128(a_src, a_off[p], kbytes, 0);
       rw[p] = __builtin_amdgcn_raw_buffer_load_b128(w_src, w_off[p], kbytes, 0);
     }
@@ -254,45 +327,37 @@ __global__ __launch_bounds__(256) void gemm_mfma_big_kernel(void* __restrict__ C
   };
   auto store_slab = [&](int buf) {
 #pragma unroll
-    for (int p = 0; p < 8; ++p) {
-      const int off = (lrow + 32 * p) * LDS_ROW + lchunk * 8;
+    for (int p = 0; p < 4; ++p) {
+      const int off = (lrow + 64 * p) * LDS_ROW + lchunk * 8;
       *reinterpret_cast<u32x4_t*>(As + buf * BIG_TILE_ELEMS + off) = ra[p];
       *reinterpret_cast<u32x4_t*>(Ws + buf * BIG_TILE_ELEMS + off) = rw[p];
     }
   };
 
-  f32x16_t acc[4][4];
+  f32x16_t acc[4][2];
 #pragma unroll
   for (int i = 0; i < 4; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j)
+    for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   const int frow = lane % 32, fk = (lane / 32) * 8;
-  Frag fa[2][4], fb[2][4];
+  Frag fa[2][4], fb[2][2];
   auto read_frags = [&](int which, int buf, int ks) {   // ks: which 16 k of the slab
     const uint16_t* a_base = As + buf * BIG_TILE_ELEMS + (wm * 128 + frow) * LDS_ROW + fk + ks * 16;
-    const uint16_t* w_base = Ws + buf * BIG_TILE_ELEMS + (wn * 128 + frow) * LDS_ROW + fk + ks * 16;
+    const uint16_t* w_base = Ws + buf * BIG_TILE_ELEMS + (wn * 64 + frow) * LDS_ROW + fk + ks * 16;
 #pragma unroll
     for (int i = 0; i < 4; ++i) fa[which][i].n = *reinterpret_cast<const u32x4_t*>(a_base + i * 32 * LDS_ROW);
 #pragma unroll
-    for (int j = 0; j < 4; ++j) fb[which][j].n = *reinterpret_cast<const u32x4_t*>(w_base + j * 32 * LDS_ROW);
+    for (int j = 0; j < 2; ++j) fb[which][j].n = *reinterpret_cast<const u32x4_t*>(w_base + j * 32 * LDS_ROW);
   };
   auto products = [&](int which) {
 #pragma unroll
     for (int i = 0; i < 4; ++i)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[i][j] = mfma32(fa[which][i], fb[which][j], acc[i][j]);
+      for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(fa[which][i], fb[which][j], acc[i][j]);
   };
-  // the order wanted inside one scheduling region: one matrix-core instruction, then one of
-  // each kind of memory instruction named, `n` times; the rest of the 16 after that
-#define PI_DEAL(n, kind_a, kind_b)                                                   \
-  _Pragma("unroll") for (int d_ = 0; d_ < n; ++d_) {                                 \
-    __builtin_amdgcn_sched_group_barrier(PI_SCHED_MFMA, 1, 0);                       \
-    if (kind_a) __builtin_amdgcn_sched_group_barrier(kind_a, 1, 0);                  \
-    if (kind_b) __builtin_amdgcn_sched_group_barrier(kind_b, 1, 0);                  \
-  }
 
   load_slab(0);
   store_slab(0);
@@ -303,65 +368,29 @@ __global__ __launch_bounds__(256) void gemm_mfma_big_kernel(void* __restrict__ C
     const int buf = s & 1;
     read_frags(1, buf, 1);
     products(0);
-    PI_DEAL(8, PI_SCHED_DS_READ, 0)
-    PI_DEAL(8, 0, 0)
     read_frags(0, buf, 2);
     products(1);
-    PI_DEAL(8, PI_SCHED_DS_READ, 0)
-    PI_DEAL(8, 0, 0)
     read_frags(1, buf, 3);
     products(0);
     store_slab(buf ^ 1);            // slab s + 1, loaded during the previous slab's last step
-    PI_DEAL(8, PI_SCHED_DS_READ, PI_SCHED_DS_WRITE)
-    PI_DEAL(8, PI_SCHED_DS_WRITE, 0)
     __syncthreads();
     load_slab(s + 2);
     read_frags(0, buf ^ 1, 0);
     products(1);
-    PI_DEAL(8, PI_SCHED_VMEM_READ, PI_SCHED_DS_READ)
-    PI_DEAL(8, PI_SCHED_VMEM_READ, 0)
   }
-#undef PI_DEAL
 
-  // acc[i][j][v] is C[m0 + wm*128 + i*32 + 8*(v/4) + 4*(lane/32) + v%4][n0 + wn*128 + j*32 + lane%32].
-  // Offsets inside the wave's 128 x 128 corner are 32-bit (the host checks 128 * ldc fits).
-  const int half = lane / 32, ccol = lane % 32;
-  const long mw = m0 + wm * 128, nw = n0 + wn * 128;
-  const int rows_left = (int)min((long)128, M - mw), cols_left = (int)min((long)128, N - nw);   // may be <= 0
-  const int ld = (int)ldc;
-  if (EPI == EPI_SWIGLU) {
-    // columns 0..15 of a tile are gate rows of W, 16..31 the up rows of the same features: bring
-    // the two together (the swap leaves the gate value in both 16-lane rows of one result and
-    // the up value in both rows of the other); the lower rows store
-    bf16_t* C = reinterpret_cast<bf16_t*>(Cv) + mw * ldc + nw / 2;
+  // acc[i][j][v] is C[m0 + wm*128 + i*32 + 8*(v/4) + 4*(lane/32) + v%4][n0 + wn*64 + j*32 + lane%32].
+  // Offsets inside the wave's corner are 32-bit (the host checks that 128 * ldc fits).
+  __syncthreads();                              // LDS is free for the waves' patches
+  {
+    const long mw = m0 + wm * 128, nw = n0 + wn * 64;
+    const int rows_left = (int)min((long)128, M - mw), cols_left = (int)min((long)64, N - nw);   // may be <= 0
+    float* patch = reinterpret_cast<float*>(lds) + wave * PATCH_FLOATS;
+    const int esize = EPI == EPI_BF16 || EPI == EPI_SWIGLU ? 2 : 4;
+    char* corner = reinterpret_cast<char*>(Cv) + (mw * ldc + (EPI == EPI_SWIGLU ? nw / 2 : nw)) * esize;
+    const bool wide = (ldc * esize) % 16 == 0 && reinterpret_cast<uintptr_t>(corner) % 16 == 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-#if defined(__HIP_DEVICE_COMPILE__)
-          const unsigned bits = __float_as_uint(acc[i][j][v]);
-          auto gu = __builtin_amdgcn_permlane16_swap(bits, bits, false, false);
-          const int rl = i * 32 + 8 * (v / 4) + 4 * half + v % 4;
-          if (ccol < 16 && rl < rows_left && j * 32 + ccol + 16 < cols_left)
-            C[rl * ld + j * 16 + ccol] = from_float<bf16_t>(silu_mul(__uint_as_float(gu[0]), __uint_as_float(gu[1])));
-#endif
-        }
-  } else {
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-          const int rl = i * 32 + 8 * (v / 4) + 4 * half + v % 4, cl = j * 32 + ccol;
-          if (rl >= rows_left || cl >= cols_left) continue;
-          const int off = rl * ld + cl;
-          if (EPI == EPI_BF16) (reinterpret_cast<bf16_t*>(Cv) + mw * ldc + nw)[off] = from_float<bf16_t>(acc[i][j][v]);
-          if (EPI == EPI_F32) (reinterpret_cast<float*>(Cv) + mw * ldc + nw)[off] = acc[i][j][v];
-          if (EPI == EPI_ACCUM) (reinterpret_cast<float*>(Cv) + mw * ldc + nw)[off] += acc[i][j][v];
-        }
+    for (int i = 0; i < 4; ++i) store_rows32<EPI>(patch, acc[i][0], acc[i][1], corner, (int)ldc, i * 32, rows_left, cols_left, lane, wide);
   }
 }
 
@@ -384,7 +413,7 @@ static int launch(void* C, long ldc, const void* A, long lda, const void* W, lon
   kps = ((kps + BK - 1) / BK) * BK;
   splits = ceil_div(K, kps);
   const long big_tiles = (long)ceil_div(M, GM) * ceil_div(N, GN);
-  if (big_tiles * splits >= BIG_MIN_TILES && big_tiles < 2147483647L && ldc < (1L << 23) && K % BK == 0) {
+  if (big_tiles * splits >= BIG_MIN_TILES && big_tiles < 2147483647L && K % BK == 0) {
     static bool big_configured = false;
     if (!big_configured) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma_big_kernel<EPI>),
@@ -392,7 +421,7 @@ static int launch(void* C, long ldc, const void* A, long lda, const void* W, lon
       if (e != hipSuccess) return pi_fail("gemm_mfma: cannot reserve %zu bytes of LDS: %s", kBigLdsBytes, hipGetErrorString(e));
       big_configured = true;
     }
-    hipLaunchKernelGGL((gemm_mfma_big_kernel<EPI>), dim3((unsigned)big_tiles, splits), dim3(256), kBigLdsBytes, stream, C, ldc,
+    hipLaunchKernelGGL((gemm_mfma_big_kernel<EPI>), dim3((unsigned)big_tiles, splits), dim3(512), kBigLdsBytes, stream, C, ldc,
                        (const bf16_t*)A, lda, (const bf16_t*)W, ldw, M, N, K, ceil_div(N, GN), kps);
     return pi_check_launch("gemm_mfma_big");
   }
@@ -420,6 +449,7 @@ extern "C" int pi_gemm_mfma(void* C, int epilogue, long ldc, const void* A, long
              "gemm_mfma: a k-split (%d) needs the float32 store into a [splits, M, N] workspace", splits);
   PI_REQUIRE(K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0, "gemm_mfma: K (%d) and row strides (%ld, %ld) must be multiples of 8", K, lda, ldw);
   PI_REQUIRE(256 * lda < (1L << 29) && 256 * ldw < (1L << 29), "gemm_mfma: row strides (%ld, %ld) are too long for 32-bit offsets inside a tile", lda, ldw);
+  PI_REQUIRE(ldc > 0 && ldc < (1L << 23), "gemm_mfma: the result's row stride (%ld) is too long for 32-bit offsets inside a tile", ldc);
   PI_REQUIRE(((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_mfma: operands must be 16-byte aligned");
   PI_REQUIRE(epilogue != EPI_SWIGLU || N % 32 == 0, "gemm_mfma: the SwiGLU epilogue needs N (%d) to be a multiple of 32", N);
   PI_REQUIRE((long)ceil_div(M, BM) * ceil_div(N, BN) < 2147483647L, "gemm_mfma: too many tiles");
