@@ -364,20 +364,37 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
   __syncthreads();
   load_slab(1);
   read_frags(0, 0, 0);
+  // the order wanted inside one scheduling region: one matrix-core instruction, then one of
+  // each kind of memory instruction named, `n` times; the rest of the 8 after that
+#define PI_DEAL(n, kind_a, kind_b)                                                   \
+  _Pragma("unroll") for (int d_ = 0; d_ < n; ++d_) {                                 \
+    __builtin_amdgcn_sched_group_barrier(PI_SCHED_MFMA, 1, 0);                       \
+    if (kind_a) __builtin_amdgcn_sched_group_barrier(kind_a, 1, 0);                  \
+    if (kind_b) __builtin_amdgcn_sched_group_barrier(kind_b, 1, 0);                  \
+  }
   for (int s = 0; s < slabs; ++s) {
     const int buf = s & 1;
     read_frags(1, buf, 1);
     products(0);
+    PI_DEAL(6, PI_SCHED_DS_READ, 0)
+    PI_DEAL(2, 0, 0)
     read_frags(0, buf, 2);
     products(1);
+    PI_DEAL(6, PI_SCHED_DS_READ, 0)
+    PI_DEAL(2, 0, 0)
     read_frags(1, buf, 3);
     products(0);
     store_slab(buf ^ 1);            // slab s + 1, loaded during the previous slab's last step
+    PI_DEAL(6, PI_SCHED_DS_READ, PI_SCHED_DS_WRITE)
+    PI_DEAL(2, PI_SCHED_DS_WRITE, 0)
     __syncthreads();
     load_slab(s + 2);
     read_frags(0, buf ^ 1, 0);
     products(1);
+    PI_DEAL(6, PI_SCHED_VMEM_READ, PI_SCHED_DS_READ)
+    PI_DEAL(2, PI_SCHED_VMEM_READ, 0)
   }
+#undef PI_DEAL
 
   // acc[i][j][v] is C[m0 + wm*128 + i*32 + 8*(v/4) + 4*(lane/32) + v%4][n0 + wn*64 + j*32 + lane%32].
   // Offsets inside the wave's corner are 32-bit (the host checks that 128 * ldc fits).
