@@ -32,7 +32,7 @@ SHARED_TARGET_BLOCKS = 256     # ... and this many blocks wanted (one per comput
 GEMM_PART_FLOATS = 16 << 20    # workspace for the pieces of products split over k (64 MB)
 TILE_MAX_SPLITS = 4
 ATTN_PART_FLOATS = 4 << 20     # key-split partial results of decode attention
-MAX_DECODE_SPLITS = 32
+MAX_DECODE_SPLITS = 64         # the combine kernel holds one key range per lane
 DECODE_WAVES_WANTED = 1024     # waves of the decode attention kernel that fill the chip (measured: flat from 512 to 1024, worse beyond)
 DECODE_MIN_KEYS_PER_SPLIT = 128
 
