@@ -6,8 +6,9 @@
 Prints ONE JSON line.  ``value`` is decoded tokens per second at batch 8 with the context
 length of the benchmark configuration (every request's cache holds that many tokens when
 the timed steps end).  A "step" is one decode step of the whole batch through the engine's
-own path: metadata upload, the replayed graph (model + sampling kernel), and the copy of the
-chosen tokens back to the host, which the next step waits for.
+own path, driven as the engine drives its decode phase: metadata upload, the replayed graph
+(model + sampling kernel) that takes its tokens from the step before it on the device, and
+the copy of the chosen tokens to the host, which reads every step's tokens one step late.
 Also on the line: ``prefill`` (one 2,048-token prompt in one step), ``roofline`` (bytes the
 decode step has to read / its time, against 8 TB/s) and ``points`` (batch 1 and 64).
 Weights are random (N(0, 0.02), norms 1), token ids uniform random; no dataset is involved.
@@ -116,17 +117,29 @@ def time_decode(runner, batch, steps, warmup, context, seed=1, synthetic_cache=F
             lc.v.normal_()
     last = torch.randint(0, vocab, (batch,), generator=g).tolist()
     temps, draws = [0.0] * batch, [0.0] * batch
+    rows = list(range(batch))
+    host = [torch.empty(batch, dtype=torch.int32, pin_memory=True) for _ in range(2)]
+    arrived = [torch.cuda.Event(), torch.cuda.Event()]
 
-    def one_step(tokens):
-        out = runner.decode_step([StepEntry(rid, [t], [0]) for rid, t in zip(rids, tokens)], temps, draws)
-        return out.tolist()       # the next step needs these: the copy back is part of the step
+    # The loop of the engine's decode phase: a step takes its tokens from the step before it on
+    # the device, and the host reads a step's tokens while the next one runs (one step late).
+    def run(n, ids):
+        for i in range(n):
+            if ids is None:
+                ids = runner.decode_step([StepEntry(rid, [t], [0]) for rid, t in zip(rids, last)], temps, draws)
+            else:
+                ids = runner.decode_step([StepEntry(rid, [0], [0]) for rid in rids], temps, draws, (ids, rows))
+            host[i % 2].copy_(ids, non_blocking=True)
+            arrived[i % 2].record()
+            if i:
+                arrived[(i - 1) % 2].synchronize()
+                host[(i - 1) % 2].tolist()
+        return ids
 
-    for _ in range(warmup):
-        last = one_step(last)
+    ids = run(warmup, None)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        last = one_step(last)
+    run(steps, ids)
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     mean_ctx = context - (steps - 1) / 2.0        # keys each request reads, averaged over the timed steps
