@@ -39,6 +39,18 @@ struct KVChunk {
   Frag k[2][HD / 32];   // key tiles: rows key0 + lane % 16
   Frag v[HD / 16];      // value rows d = db*16 + lane % 16; keys (lane/16)*4..+3 of both tiles
   bool have[2];
+  __device__ inline Frag key(int t, int ks) const { return k[t][ks]; }
+  __device__ inline Frag val(int db) const { return v[db]; }
+};
+
+// The same chunk lying in LDS in operand order ([fragment][lane], keys first): a fragment is
+// read when the arithmetic wants it, so that a chunk never occupies registers as a whole.
+template <int HD>
+struct StagedChunk {
+  const u32x4_t* from;  // this lane's first fragment
+  bool have[2];
+  __device__ inline Frag key(int t, int ks) const { Frag f; f.n = from[(t * (HD / 32) + ks) * 64]; return f; }
+  __device__ inline Frag val(int db) const { Frag f; f.n = from[(HD / 16 + db) * 64]; return f; }
 };
 
 template <int HD, int CB>
@@ -148,8 +160,8 @@ __device__ inline void attn_load(KVChunk<HD>& kv, const ChunkPages& cp, const bf
 // st.m is a column's reference score (raw, before the softmax scale): at least the largest
 // score seen minus the slack.  Moving it costs a pass over the accumulators, so it only moves
 // when some column of the wave needs it.
-template <int HD, int CB, bool MASKED>
-__device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv, int k0, float scale_log2, int lane) {
+template <int HD, int CB, bool MASKED, class KV>
+__device__ inline void attn_compute(AttnState<HD, CB>& st, const KV& kv, int k0, float scale_log2, int lane) {
   const int lg = lane / 16;
   f32x4_t s[2][CB];
 #pragma unroll
@@ -158,7 +170,7 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv
     for (int c = 0; c < CB; ++c) {
       f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < HD / 32; ++ks) acc = mfma16(kv.k[t][ks], st.q[c][ks], acc);
+      for (int ks = 0; ks < HD / 32; ++ks) acc = mfma16(kv.key(t, ks), st.q[c][ks], acc);
       s[t][c] = acc;
     }
   const float slack = PI_RESCALE_SLACK / scale_log2;
@@ -210,7 +222,7 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv
     pb.q.w = pack_bf16x2(p[1][2], p[1][3]);
 #pragma unroll
     for (int db = 0; db < HD / 16; ++db) {
-      Frag va = kv.v[db];
+      Frag va = kv.val(db);
       if (MASKED) {   // a missing tile was read from page 0: its values must not meet even a zero weight
         if (!kv.have[0]) va.d[0] = make_uint2(0u, 0u);
         if (!kv.have[1]) va.d[1] = make_uint2(0u, 0u);
@@ -220,11 +232,10 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv
   }
 }
 
-template <int HD, int CB>
-__device__ inline void attn_compute(AttnState<HD, CB>& st, const KVChunk<HD>& kv, int k0, float scale_log2, bool masked,
-                                    int lane) {
-  if (masked) attn_compute<HD, CB, true>(st, kv, k0, scale_log2, lane);
-  else attn_compute<HD, CB, false>(st, kv, k0, scale_log2, lane);
+template <int HD, int CB, class KV>
+__device__ inline void attn_compute(AttnState<HD, CB>& st, const KV& kv, int k0, float scale_log2, bool masked, int lane) {
+  if (masked) attn_compute<HD, CB, true, KV>(st, kv, k0, scale_log2, lane);
+  else attn_compute<HD, CB, false, KV>(st, kv, k0, scale_log2, lane);
 }
 
 // Walk chunks c0 .. c1-1 (32 keys each) with the next chunk's loads in flight during the

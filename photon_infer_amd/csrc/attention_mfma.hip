@@ -112,18 +112,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
         for (int j = 0; j < 4; ++j) {
           const int key0 = sc * KEYS_PER_ROUND + j * 32;
           if (key0 > see_any_hi || key0 + 31 < see_any_lo) continue;
-          KVChunk<HD> kv;
-          const u32x4_t* from = staged + ((buf * 4 + j) * F) * 64 + lane;
-#pragma unroll
-          for (int t = 0; t < 2; ++t)
-#pragma unroll
-            for (int ks = 0; ks < HD / 32; ++ks) kv.k[t][ks].n = from[(t * (HD / 32) + ks) * 64];
-#pragma unroll
-          for (int db = 0; db < HD / 16; ++db) kv.v[db].n = from[(HD / 16 + db) * 64];
+          StagedChunk<HD> kv;
+          kv.from = staged + ((buf * 4 + j) * F) * 64 + lane;
           kv.have[0] = __builtin_amdgcn_readfirstlane(present[buf][j][0]) != 0;
           kv.have[1] = __builtin_amdgcn_readfirstlane(present[buf][j][1]) != 0;
           const bool masked = key0 < see_all_lo || key0 + 31 > see_all_hi || !kv.have[0] || !kv.have[1];
-          attn_compute<HD, CB>(st, kv, key0, scale_log2, masked, lane);
+          attn_compute<HD, CB, StagedChunk<HD>>(st, kv, key0, scale_log2, masked, lane);
         }
       }
       stash(buf ^ 1);

@@ -42,6 +42,12 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
 ]
+# Per file: the prompt-attention kernel keeps its matrix-core accumulators in ordinary vector
+# registers.  In the accumulator registers the allocator moved them between register tuples
+# from one matrix instruction to the next (hundreds of copies per 32 keys at head size 128).
+FILE_FLAGS: Dict[str, List[str]] = {
+    "attention_mfma.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"],
+}
 
 
 def _log(msg: str) -> None:
@@ -84,6 +90,7 @@ def source_hash(module: str) -> str:
     host = module in HOST_MODULES
     h = hashlib.sha256(" ".join(HOST_FLAGS if host else HIPCC_FLAGS).encode())
     for name in MODULES[module] + ([] if host else HEADERS):
+        h.update(" ".join(FILE_FLAGS.get(name, [])).encode())
         path = os.path.join(CSRC_DIR, name)
         if os.path.isfile(path):
             with open(path, "rb") as f:
@@ -148,7 +155,7 @@ def build_module(module: str, force: bool = False, quiet: bool = False) -> str:
     try:
         def compile_one(src: str) -> str:
             obj = os.path.join(bdir, f"{module}_{os.path.splitext(os.path.basename(src))[0]}.{os.getpid()}.o")
-            _run([hipcc, *compile_flags, "-I", CSRC_DIR, "-c", os.path.join(CSRC_DIR, src), "-o", obj], src)
+            _run([hipcc, *compile_flags, *FILE_FLAGS.get(src, []), "-I", CSRC_DIR, "-c", os.path.join(CSRC_DIR, src), "-o", obj], src)
             if not quiet:
                 _log(f"  compiled {src} ({time.time() - t0:.0f} s)")
             return obj
