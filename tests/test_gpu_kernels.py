@@ -374,7 +374,9 @@ def test_attention_finds_one_far_key_among_hundreds(_ops, dtype, fast):
     nh, nkv, hd, page = 4, 2, 64, 16
     g = gen(11)
     for kv_len, q_len, hot in [(777, 1, 3), (777, 1, 776), (640, 1, 639), (777, 1, 512), (500, 37, 15), (500, 37, 463),
-                               (129, 2, 127)]:
+                               (129, 2, 127),
+                               # one long request: the decode kernel cuts it into its largest number of key ranges
+                               (9000, 1, 5), (9000, 1, 4417), (9000, 1, 8999)]:
         k = torch.randn(kv_len, nkv, hd, generator=g) * 0.1
         v = torch.randn(kv_len, nkv, hd, generator=g)
         q = torch.randn(q_len, nh, hd, generator=g) * 0.1
