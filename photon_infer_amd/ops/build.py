@@ -155,7 +155,15 @@ def build_module(module: str, force: bool = False, quiet: bool = False) -> str:
     try:
         def compile_one(src: str) -> str:
             obj = os.path.join(bdir, f"{module}_{os.path.splitext(os.path.basename(src))[0]}.{os.getpid()}.o")
-            _run([hipcc, *compile_flags, *FILE_FLAGS.get(src, []), "-I", CSRC_DIR, "-c", os.path.join(CSRC_DIR, src), "-o", obj], src)
+            base = [hipcc, *compile_flags, "-I", CSRC_DIR, "-c", os.path.join(CSRC_DIR, src), "-o", obj]
+            extra = [] if host else FILE_FLAGS.get(src, [])
+            try:
+                _run(base + extra, src)
+            except KernelLibraryMissing:
+                if not extra:
+                    raise
+                _log(f"  {src}: the compiler refused {' '.join(extra)}; compiling without (slower kernel, same results)")
+                _run(base, src)
             if not quiet:
                 _log(f"  compiled {src} ({time.time() - t0:.0f} s)")
             return obj
