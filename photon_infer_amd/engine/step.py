@@ -191,6 +191,11 @@ class ModelRunner:
         self.cache.commit_step(slots, [len(e.tokens) for e in entries])
         return logits
 
+    def graph_pool(self):
+        if getattr(self, "_graph_pool", None) is None:
+            self._graph_pool = torch.cuda.graph_pool_handle()
+        return self._graph_pool
+
     @torch.no_grad()
     def decode_step(self, entries: Sequence[StepEntry], temperatures: Sequence[float], uniforms: Sequence[float],
                     feed: Optional[Tuple[torch.Tensor, Sequence[int]]] = None) -> torch.Tensor:
@@ -273,6 +278,7 @@ class _DecodeGraph:
             h["logit_rows"][:] = np.arange(R)
             h["q_start"][:] = np.arange(R + 1)
             self._staging.append((host, h, hf))
+        self._copied = [torch.cuda.Event(), torch.cuda.Event()]    # a staging buffer's last copy to the device
         self._turn = 0
         self.host, self.h, self.hf = self._staging[0]
         self.dev = torch.zeros(total, dtype=torch.int32, device=runner.device)
@@ -292,6 +298,7 @@ class _DecodeGraph:
         cache = self.runner.cache
         self._turn ^= 1
         self.host, self.h, self.hf = self._staging[self._turn]
+        self._copied[self._turn].synchronize()      # a caller more than one step ahead waits here, not corrupts
         if feed is None:
             self.h["token_ids"][:] = [e.tokens[0] for e in entries]
         else:
@@ -305,6 +312,7 @@ class _DecodeGraph:
             self.h[f"table{g}"].reshape(self.R, self.width)[:] = cache.table_rows(g, slots, self.width)
         self.ctx.host_slots = slots
         self.dev.copy_(self.host, non_blocking=True)
+        self._copied[self._turn].record()
         if feed is not None:      # the tokens come from an earlier step's result, on the device
             torch.index_select(feed[0], 0, self.feed_rows, out=self.ctx.token_ids)
 
@@ -325,7 +333,10 @@ class _DecodeGraph:
             collecting = gc.isenabled()
             gc.disable()
             try:
-                with torch.cuda.graph(graph):
+                # all graphs of a runner take their intermediate buffers from one pool: they
+                # never run at the same time and hold nothing in it between replays (the
+                # sampled tokens and the metadata lie outside)
+                with torch.cuda.graph(graph, pool=self.runner.graph_pool()):
                     self._body()
             finally:
                 if collecting:

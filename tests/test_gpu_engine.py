@@ -217,3 +217,36 @@ def test_an_end_token_during_a_step_ahead(tmp_path):
     for i in (0, 2):                       # the others run on unless they meet the token themselves
         n = free[i].index(stop) + 1 if stop in free[i] else 12
         assert ahead[i] == free[i][:n]
+
+
+def test_decode_steps_queued_far_ahead_of_the_gpu(tmp_path):
+    """A caller may queue several decode steps without reading any result while the GPU is
+    still busy with earlier work: every step must still see its own positions and tables
+    (the metadata staging is reused only after its copy has run)."""
+    from photon_infer_amd.engine import StepEntry
+
+    d = make_model_dir(tmp_path, "D", seed=37)
+    vocab = ALL["D"][0]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 60 + n) for n in (5, 18, 11)]
+    fed = [random_tokens(7, vocab, 50 + i) for i in range(3)]          # the tokens fed at each decode step, fixed
+
+    def run(busy):
+        runner = engine(d, "D", dtype="bfloat16").runner
+        rids = [f"r{i}" for i in range(3)]
+        for rid, p in zip(rids, prompts):
+            runner.admit(rid)
+            runner.step([StepEntry(rid, p, [])])
+        outs = []
+        for s in range(7):
+            if s == 1:                                                 # step 0 captured the graph (and drained the GPU)
+                torch.cuda.synchronize()
+                if busy:
+                    torch.cuda._sleep(400_000_000)                     # the GPU stays behind the host for a while
+            ids = runner.decode_step([StepEntry(rid, [fed[i][s]], [0]) for i, rid in enumerate(rids)], [0.0] * 3, [0.0] * 3)
+            outs.append(ids.clone())
+            if not busy:
+                torch.cuda.synchronize()
+        torch.cuda.synchronize()
+        return [o.tolist() for o in outs]
+
+    assert run(True) == run(False)
