@@ -211,36 +211,66 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   const int slabs = (k_hi - k_lo + BK - 1) / BK;
-  load_slab(0);
-  store_slab(0);
-  __syncthreads();
   // 32 x 32 x 16 instruction: a lane reads row lane % 32, 16 bytes at k = (lane / 32) * 8; with
   // rows 144 bytes apart the 16 lanes served together fall on distinct banks
   const int frow = lane % 32, fk = (lane / 32) * 8;
+  Frag fa[2][2], fb[2][2];
+  auto read_frags = [&](int which, int buf, int ks) {   // ks: which 16 k of the slab
+    const uint16_t* a_base = As + buf * TILE_ELEMS + (wm * 64 + frow) * LDS_ROW + fk + ks * 16;
+    const uint16_t* w_base = Ws + buf * TILE_ELEMS + (wn * 64 + frow) * LDS_ROW + fk + ks * 16;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) fa[which][i].n = *reinterpret_cast<const u32x4_t*>(a_base + i * 32 * LDS_ROW);
+#pragma unroll
+    for (int j = 0; j < 2; ++j) fb[which][j].n = *reinterpret_cast<const u32x4_t*>(w_base + j * 32 * LDS_ROW);
+  };
+  auto products = [&](int which) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(fa[which][i], fb[which][j], acc[i][j]);
+  };
+  // The loop has no branch: a slab beyond the range loads zeros (offsets out of the
+  // descriptor's range) into the buffer nobody reads.  Fragments of the next 16 k are read
+  // while the matrix instructions of these 16 run; the hints deal one memory instruction of
+  // each kind named after every matrix instruction.
+#define PI_SCHED_MFMA 0x008
+#define PI_SCHED_VMEM_READ 0x020
+#define PI_SCHED_DS_READ 0x100
+#define PI_SCHED_DS_WRITE 0x200
+#define PI_DEAL4(kind_a, kind_b)                                                     \
+  _Pragma("unroll") for (int d_ = 0; d_ < 4; ++d_) {                                 \
+    __builtin_amdgcn_sched_group_barrier(PI_SCHED_MFMA, 1, 0);                       \
+    if (kind_a) __builtin_amdgcn_sched_group_barrier(kind_a, 1, 0);                  \
+    if (kind_b) __builtin_amdgcn_sched_group_barrier(kind_b, 2, 0);                  \
+  }
+  load_slab(0);
+  store_slab(0);
+  __syncthreads();
+  load_slab(BK);
+  read_frags(0, 0, 0);
   for (int s = 0; s < slabs; ++s) {
     const int buf = s & 1;
-    if (s + 1 < slabs) load_slab((s + 1) * BK);
-    const uint16_t* a_base = As + buf * TILE_ELEMS + (wm * 64 + frow) * LDS_ROW + fk;
-    const uint16_t* w_base = Ws + buf * TILE_ELEMS + (wn * 64 + frow) * LDS_ROW + fk;
-#pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      Frag a[2], b[2];
-#pragma unroll
-      for (int i = 0; i < 2; ++i) a[i].n = *reinterpret_cast<const u32x4_t*>(a_base + i * 32 * LDS_ROW + ks * 16);
-#pragma unroll
-      for (int j = 0; j < 2; ++j) b[j].n = *reinterpret_cast<const u32x4_t*>(w_base + j * 32 * LDS_ROW + ks * 16);
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(a[i], b[j], acc[i][j]);
-    }
-    if (s + 1 < slabs) store_slab(buf ^ 1);
+    read_frags(1, buf, 1);
+    products(0);
+    PI_DEAL4(PI_SCHED_DS_READ, 0)
+    read_frags(0, buf, 2);
+    products(1);
+    PI_DEAL4(PI_SCHED_DS_READ, 0)
+    read_frags(1, buf, 3);
+    products(0);
+    store_slab(buf ^ 1);            // slab s + 1, loaded while slab s - 1's last step ran
+    PI_DEAL4(PI_SCHED_DS_READ, PI_SCHED_DS_WRITE)
     __syncthreads();
+    load_slab((s + 2) * BK);
+    read_frags(0, buf ^ 1, 0);
+    products(1);
+    PI_DEAL4(PI_SCHED_DS_READ, PI_SCHED_VMEM_READ)
   }
+#undef PI_DEAL4
+  __syncthreads();                  // the fragments read last belong to no slab; LDS is free for the patches
 
   // acc[i][j][v] is C[m0 + wm*64 + i*32 + 8*(v/4) + 4*(lane/32) + v%4][n0 + wn*64 + j*32 + lane%32].
-  // The loop ended with a barrier, so LDS is free for the waves' patches.  Offsets inside the
-  // wave's corner are 32-bit (the host checks that 128 * ldc fits).
+  // Offsets inside the wave's corner are 32-bit (the host checks that 128 * ldc fits).
   {
     const long mw = m0 + wm * 64, nw = n0 + wn * 64;
     const int rows_left = (int)min((long)64, M - mw), cols_left = (int)min((long)64, N - nw);   // may be <= 0
@@ -269,10 +299,6 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
 #define GM 256
 #define GN 256
 #define BIG_TILE_ELEMS (GM * LDS_ROW)
-#define PI_SCHED_MFMA 0x008
-#define PI_SCHED_VMEM_READ 0x020
-#define PI_SCHED_DS_READ 0x100
-#define PI_SCHED_DS_WRITE 0x200
 
 template <int EPI>
 __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ A, long lda,
