@@ -191,8 +191,12 @@ class ContinuousBatchEngine:
         self.steps += 1
         return done
 
+    def has_work(self) -> bool:
+        """Requests waiting or running, or a launched step whose tokens have not been read."""
+        return self.scheduler.has_work() or self._in_flight is not None
+
     def run_until_complete(self, print_progress: bool = False) -> None:
-        while self.scheduler.has_work() or self._in_flight is not None:
+        while self.has_work():
             if print_progress and self.steps % 10 == 0:
                 s = self.scheduler.get_stats()
                 print(f"Step {self.steps}: Running={s.num_running} Waiting={s.num_waiting} Finished={s.num_finished}",

@@ -30,9 +30,12 @@ MODULES: Dict[str, List[str]] = {
     "bf16": ["gemm_mfma.hip", "gemm_skinny.hip", "attention_mfma.hip", "attention_decode.hip"],
     # host only: cache manager bookkeeping (needs no GPU and no hipcc)
     "runtime": ["runtime/cache.cpp"],
+    # host only: the engine for C / C++ programs (hosts an interpreter; links libpython)
+    "api": ["api/photon_engine.cpp"],
 }
 HEADERS = ["common.h", "mfma.h", "attention_mfma.h"]
-HOST_MODULES = {"runtime"}
+HOST_MODULES = {"runtime", "api"}
+HOST_HEADERS = {"api": ["api/photon_engine.h"]}
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]
 
 ARCH = "gfx950"
@@ -71,6 +74,15 @@ def _host_compiler() -> str:
                                "the runtime library cannot be built")
 
 
+def python_embed_flags():
+    """(compile flags, link flags) for a program or library that hosts this interpreter."""
+    import sysconfig
+    inc = sysconfig.get_paths()["include"]
+    libdir = sysconfig.get_config_var("LIBDIR") or "/usr/lib"
+    version = sysconfig.get_config_var("LDVERSION") or sysconfig.get_python_version()
+    return [f"-I{inc}"], [f"-L{libdir}", f"-Wl,-rpath,{libdir}", f"-lpython{version}", "-ldl"]
+
+
 def _build_dir() -> str:
     d = os.path.join(CSRC_DIR, "_build")
     try:
@@ -89,7 +101,7 @@ def _build_dir() -> str:
 def source_hash(module: str) -> str:
     host = module in HOST_MODULES
     h = hashlib.sha256(" ".join(HOST_FLAGS if host else HIPCC_FLAGS).encode())
-    for name in MODULES[module] + ([] if host else HEADERS):
+    for name in MODULES[module] + (HOST_HEADERS.get(module, []) if host else HEADERS):
         h.update(" ".join(FILE_FLAGS.get(name, [])).encode())
         path = os.path.join(CSRC_DIR, name)
         if os.path.isfile(path):
@@ -134,6 +146,10 @@ def build_module(module: str, force: bool = False, quiet: bool = False) -> str:
     hipcc = _host_compiler() if host else _hipcc()
     compile_flags = HOST_FLAGS if host else HIPCC_FLAGS
     link_flags = ["-shared", "-fPIC"] if host else [f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc"]
+    link_libs: List[str] = []
+    if module == "api":
+        compile_flags = compile_flags + python_embed_flags()[0]
+        link_libs = python_embed_flags()[1]
     bdir = _build_dir()
     sources = MODULES[module]
     missing = [s for s in sources if not os.path.isfile(os.path.join(CSRC_DIR, s))]
@@ -171,7 +187,7 @@ def build_module(module: str, force: bool = False, quiet: bool = False) -> str:
         with ThreadPoolExecutor(max_workers=min(8, len(sources))) as pool:
             objs = list(pool.map(compile_one, sources))
         tmp = f"{lib}.{os.getpid()}.tmp"
-        _run([hipcc, *link_flags, *objs, "-o", tmp], f"libphoton_{module}.so")
+        _run([hipcc, *link_flags, *objs, *link_libs, "-o", tmp], f"libphoton_{module}.so")
         os.replace(tmp, lib)
         with open(lib + ".hash", "w") as f:
             f.write(source_hash(module))

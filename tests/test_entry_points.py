@@ -33,3 +33,14 @@ def test_graft_entry_has_build_and_smoke():
     finally:
         sys.path.pop(0)
     assert callable(entry.build) and callable(entry.smoke)
+
+
+def test_cpp_program_reports_a_missing_model_folder(tmp_path):
+    """The library API for C++ programs builds, links and turns an engine error into an exception."""
+    import cpp_api
+
+    exe = cpp_api.build_demo(tmp_path)
+    r = cpp_api.run_demo(exe, tmp_path / "no_such_model", "float32", "1,2,3", 4)
+    assert r.returncode == 3, (r.stdout, r.stderr)
+    # without a GPU the engine refuses before it looks at the folder; with one it names the folder
+    assert "engine error:" in r.stderr and ("no_such_model" in r.stderr or "GPU" in r.stderr)

@@ -250,3 +250,18 @@ def test_decode_steps_queued_far_ahead_of_the_gpu(tmp_path):
         return [o.tolist() for o in outs]
 
     assert run(True) == run(False)
+
+
+def test_cpp_program_generates_what_the_python_entry_point_generates(model_dirs, tmp_path):
+    """The library API for C and C++ programs drives the same engine: a C++ program built
+    against it generates the same tokens for the same requests."""
+    import cpp_api
+
+    prompts = [random_tokens(n, 256, 40 + n) for n in (5, 12, 3)]
+    want = engine(model_dirs["A"], "A").generate(prompts, max_new_tokens=9, ignore_eos=True)
+    exe = cpp_api.build_demo(tmp_path)
+    r = cpp_api.run_demo(exe, model_dirs["A"], "float32", ";".join(",".join(map(str, p)) for p in prompts), 9,
+                         ALL["A"][1]["block_size"])
+    assert r.returncode == 0, (r.stdout, r.stderr)
+    got = [[int(t) for t in line.split()] for line in r.stdout.strip().splitlines()]
+    assert got == want
