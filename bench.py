@@ -24,7 +24,7 @@ import time
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
-# layer sizes of Llama 3.2 1B (BASELINE.json configs[2])
+# layer sizes of Llama 3.2 1B, the benchmark configuration
 MODEL = dict(
     architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=8192, num_hidden_layers=16,
     num_attention_heads=32, num_key_value_heads=8, head_dim=64, vocab_size=128256,

@@ -27,7 +27,7 @@ def engine(model_dir, name, **kw):
 
 
 def test_greedy_generation_equals_the_plain_implementation(model_dirs):
-    # BASELINE workload of the first tiny model: prompts of 5, 9 and 17 tokens, 8 greedy tokens each
+    # the first tiny benchmark workload: prompts of 5, 9 and 17 tokens, 8 greedy tokens each
     cfg, W = P.read_model_folder(model_dirs["A"])
     prompts = [random_tokens(n, 256, 30 + n) for n in (5, 9, 17)]
     want = [P.greedy_generate(cfg, W, p, 8) for p in prompts]
@@ -55,7 +55,7 @@ def test_greedy_generation_in_bfloat16_follows_the_plain_arg_max(model_dirs):
 
 
 def test_chunked_prefill_beside_decodes_with_temperature(model_dirs):
-    # BASELINE workload of the second tiny model: prompts 1, 7, 33, 64, 100 in 16-token chunks
+    # the second tiny benchmark workload: prompts 1, 7, 33, 64, 100 in 16-token chunks
     # beside decodes, 12 tokens each at temperature 0.8
     prompts = [random_tokens(n, 384, 50 + n) for n in (1, 7, 33, 64, 100)]
 
