@@ -14,10 +14,13 @@ template <int HD>
 __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2 : 1))) void attention_decode_kernel(
     bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q, long q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table,
-    int table_width, const int* __restrict__ q_start, const int* __restrict__ kv_len_of, int nh, int nkv, int page_size,
-    float scale, int window, long num_pages, float* __restrict__ part) {
+    int table_width, const int* __restrict__ q_start, const int* __restrict__ kv_len_of, const int* __restrict__ req_ids,
+    int nh, int nkv, int page_size, float scale, int window, long num_pages, float* __restrict__ part) {
   const int lane = threadIdx.x, lr = lane % 16, lg = lane / 16;
-  const int split = blockIdx.x, splits = gridDim.x, g = blockIdx.y, r = blockIdx.z;
+  const int split = blockIdx.x, splits = gridDim.x, g = blockIdx.y;
+  // the z-th request of this launch: all of the step's requests, or the listed ones (a step
+  // that also holds prompt portions sends only its single tokens here)
+  const int r = req_ids ? req_ids[blockIdx.z] : (int)blockIdx.z;
   const int G = nh / nkv;
   const int kv_len = kv_len_of[r];
   const int p = kv_len - 1;
@@ -60,7 +63,7 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2
   // partial: [request, head, split, HD + 4] float32: O^T (un-normalised), then m, l
   const int rec = HD + 4;   // O^T, m, l, two floats of padding (keeps 16-byte alignment)
   if (valid) {
-    float* mine = part + (((long)r * nh + head) * splits + split) * rec;
+    float* mine = part + (((long)blockIdx.z * nh + head) * splits + split) * rec;
 #pragma unroll
     for (int db = 0; db < HD / 16; ++db)
       *reinterpret_cast<f32x4_t*>(mine + db * 16 + lg * 4) = st.o[db][0];
@@ -76,11 +79,13 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2
 template <int HD>
 __global__ __launch_bounds__(64) void attention_combine_kernel(bf16_t* __restrict__ out, long out_stride,
                                                                const int* __restrict__ q_start,
+                                                               const int* __restrict__ req_ids,
                                                                const float* __restrict__ part, int nh, int splits) {
   const int lane = threadIdx.x;
-  const int head = blockIdx.x, r = blockIdx.y;
+  const int head = blockIdx.x;
+  const int r = req_ids ? req_ids[blockIdx.y] : (int)blockIdx.y;
   const int rec = HD + 4;
-  const float* base = part + ((long)r * nh + head) * splits * rec;
+  const float* base = part + ((long)blockIdx.y * nh + head) * splits * rec;
   // lane s holds range s (splits <= 64): maxima, weights and the total in parallel
   const float ms = lane < splits ? base[lane * rec + HD] : -INFINITY;
   const float ls = lane < splits ? base[lane * rec + HD + 1] : 0.f;
@@ -115,10 +120,13 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(bf16_t* __restric
 }
 
 // part: float32 [R * nh * splits * (hd + 4)], needed when splits > 1.
+// req_ids: null (requests 0 .. R-1) or the R requests of the step that this launch serves; each
+// has one query token, at row q_start[r], that sees kv_len[r] keys.
 extern "C" int pi_attention_decode(void* out, long out_stride, const void* q, long q_stride, const void* k_cache,
                                    const void* v_cache, const int* block_table, int table_width, const int* q_start,
-                                   const int* kv_len, int R, int nh, int nkv, int hd, int page_size, float scale, int window,
-                                   long num_pages, int splits, void* part, long part_elems, hipStream_t stream) {
+                                   const int* kv_len, const int* req_ids, int R, int nh, int nkv, int hd, int page_size,
+                                   float scale, int window, long num_pages, int splits, void* part, long part_elems,
+                                   hipStream_t stream) {
   PI_REQUIRE(R > 0 && nh > 0 && nkv > 0 && nh % nkv == 0 && nh / nkv <= 16, "attention_decode: needs 1..16 heads per kv head, got %d / %d", nh, nkv);
   PI_REQUIRE(hd == 64 || hd == 128, "attention_decode: head_dim %d is not 64 or 128", hd);
   PI_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_decode: page size %d must be a multiple of 16", page_size);
@@ -129,16 +137,16 @@ extern "C" int pi_attention_decode(void* out, long out_stride, const void* q, lo
   const dim3 grid(splits, nkv, R), block(64);
 #define GO(H) hipLaunchKernelGGL(attention_decode_kernel<H>, grid, block, 0, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, \
                                  q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, \
-                                 kv_len, nh, nkv, page_size, scale, window, num_pages, (float*)part)
+                                 kv_len, req_ids, nh, nkv, page_size, scale, window, num_pages, (float*)part)
   if (hd == 64) GO(64); else GO(128);
 #undef GO
   if (pi_check_launch("attention_decode")) return -1;
   if (splits > 1) {
     const dim3 cgrid(nh, R);
     if (hd == 64)
-      hipLaunchKernelGGL(attention_combine_kernel<64>, cgrid, block, 0, stream, (bf16_t*)out, out_stride, q_start, (const float*)part, nh, splits);
+      hipLaunchKernelGGL(attention_combine_kernel<64>, cgrid, block, 0, stream, (bf16_t*)out, out_stride, q_start, req_ids, (const float*)part, nh, splits);
     else
-      hipLaunchKernelGGL(attention_combine_kernel<128>, cgrid, block, 0, stream, (bf16_t*)out, out_stride, q_start, (const float*)part, nh, splits);
+      hipLaunchKernelGGL(attention_combine_kernel<128>, cgrid, block, 0, stream, (bf16_t*)out, out_stride, q_start, req_ids, (const float*)part, nh, splits);
     return pi_check_launch("attention_combine");
   }
   return 0;

@@ -208,9 +208,10 @@ def deal_tiles(walks: List[int], seats: int) -> np.ndarray:
     return order
 
 
-def _tiles(ctx, tile_rows: int, window: int, num_kv_heads: int, device):
+def _tiles(ctx, tile_rows: int, window: int, num_kv_heads: int, device, skip=()):
     """Work list of the tile kernel: (request, first token) of every tile and their deal to the
-    blocks; cached on the step (layers with the same window share it)."""
+    blocks; cached on the step (layers with the same window share it).  ``skip``: requests
+    that another kernel serves."""
     cache = getattr(ctx, "_attention_tiles", None)
     if cache is None:
         cache = {}
@@ -218,11 +219,14 @@ def _tiles(ctx, tile_rows: int, window: int, num_kv_heads: int, device):
             ctx._attention_tiles = cache
         except AttributeError:
             pass
-    key = (tile_rows, window, num_kv_heads)
+    key = (tile_rows, window, num_kv_heads, bool(skip))
     hit = cache.get(key)
     if hit is None:
         req, q0, walks = [], [], []
+        skipped = set(skip)
         for r, (n, kv) in enumerate(zip(ctx.q_lens, ctx.kv_lens)):
+            if r in skipped:
+                continue
             for start in range(0, n, tile_rows):
                 req.append(r)
                 q0.append(start)
@@ -237,6 +241,23 @@ def _tiles(ctx, tile_rows: int, window: int, num_kv_heads: int, device):
         dev = torch.from_numpy(host).to(device)
         n = len(req)
         hit = cache[key] = (dev[:n], dev[n:2 * n], dev[2 * n:], order.shape[0], seats)
+    return hit
+
+
+def _single_tokens(ctx, device):
+    """The step's requests that bring exactly one token, beside requests that bring more: their
+    indices (host tuple and device int32), cached on the step."""
+    hit = getattr(ctx, "_single_tokens", None)
+    if hit is None:
+        singles = tuple(r for r, n in enumerate(ctx.q_lens) if n == 1)
+        if len(singles) == len(ctx.q_lens):
+            singles = ()
+        ids = torch.tensor(singles, dtype=torch.int32).to(device) if singles else None
+        hit = (singles, ids)
+        try:
+            ctx._single_tokens = hit
+        except AttributeError:
+            pass
     return hit
 
 
@@ -263,20 +284,30 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
         return False
     G = num_heads // num_kv_heads
     R = ctx.R
-    if ctx.all_decode and G <= 16:
-        splits = decode_splits(R, num_kv_heads, ctx.max_kv_len)
+    def decode_kernel(n_req: int, req_ids: int, longest: int) -> None:
+        splits = decode_splits(n_req, num_kv_heads, longest)
         ws = workspace(q.device)
-        while splits > 1 and R * num_heads * splits * (head_dim + 4) > ws.attn_part.numel():
+        while splits > 1 and n_req * num_heads * splits * (head_dim + 4) > ws.attn_part.numel():
             splits -= 1
         _lib.call("bf16", "pi_attention_decode", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
                   k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
-                  ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), R, num_heads, num_kv_heads, head_dim, page_size,
-                  float(scale), int(window), pages, splits, ws.attn_part.data_ptr(), ws.attn_part.numel(), _stream())
+                  ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), req_ids, n_req, num_heads, num_kv_heads, head_dim,
+                  page_size, float(scale), int(window), pages, splits, ws.attn_part.data_ptr(), ws.attn_part.numel(),
+                  _stream())
+
+    if ctx.all_decode and G <= 16:
+        decode_kernel(R, 0, ctx.max_kv_len)
         return True
     tile_rows = attention_tile_rows(num_heads, num_kv_heads, head_dim)
     if tile_rows < 1:
         return False
-    tile_req, tile_q0, order, rounds, seats = _tiles(ctx, tile_rows, int(window), num_kv_heads, q.device)
+    # A step of prompt portions and single tokens: the single tokens, whose keys no other token
+    # of the step shares, go to the key-split kernel (a tile of one token would walk its whole
+    # context in one block, mostly on padding); the portions go to the tile kernel.
+    singles, single_ids = _single_tokens(ctx, q.device) if G <= 16 else ((), None)
+    if singles:
+        decode_kernel(len(singles), single_ids.data_ptr(), max(ctx.kv_lens[r] for r in singles))
+    tile_req, tile_q0, order, rounds, seats = _tiles(ctx, tile_rows, int(window), num_kv_heads, q.device, skip=singles)
     _lib.call("bf16", "pi_attention_prefill_mfma", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
               k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
               ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(), order.data_ptr(),

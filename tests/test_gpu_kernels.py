@@ -338,6 +338,8 @@ ATTN_CASES = [
     (8, 2, 64, 64, [130, 3, 1], [130, 250, 99], 33),                 # portions with a window, pages of 64
     (16, 1, 64, 16, [1, 1], [129, 2], None),                         # sixteen heads on one kv head
     (32, 1, 64, 16, [1, 70], [75, 70], None),                        # more heads per kv head than a wave's columns
+    (8, 2, 128, 16, [1, 70, 1, 1, 2], [900, 300, 33, 1, 50], None),  # single tokens beside portions: two kernels share the step
+    (4, 2, 64, 16, [1, 3, 1], [700, 40, 18], 25),                    # the same with a window
 ]
 
 
