@@ -33,7 +33,7 @@ GEMM_PART_FLOATS = 16 << 20    # workspace for the pieces of products split over
 TILE_MAX_SPLITS = 4
 ATTN_PART_FLOATS = 4 << 20     # key-split partial results of decode attention
 MAX_DECODE_SPLITS = 64         # the combine kernel holds one key range per lane
-DECODE_WAVES_WANTED = 1024     # waves of the decode attention kernel that fill the chip (measured: flat from 512 to 1024, worse beyond)
+DECODE_WAVES_WANTED = 512      # waves of the decode attention kernel that fill the chip (measured at batch 1 to 64: more is never faster)
 DECODE_MIN_KEYS_PER_SPLIT = 128
 
 
