@@ -1,8 +1,9 @@
-// bfloat16 matrix product for few rows (decoding: 1..64 tokens), where the weights are read
+// bfloat16 matrix product for few rows (decoding and short prompt portions: 1..128 tokens), where the weights are read
 // once from HBM and everything else is small:  C[M, N] (+)= X[M, K] . W[N, K]^T.
 //
 // The weights are the row operand of v_mfma_f32_16x16x32_bf16 and the activations the column
-// operand, so a wave produces C^T for 32 weight rows (two row tiles) and up to 64 tokens.
+// operand, so a wave produces C^T for 32 weight rows (two row tiles) and up to 32 tokens (the
+// second kernel below takes 33..128 tokens).
 // A lane reads 32 contiguous bytes of a weight row per step; the four lane groups of a row
 // cover 128 contiguous bytes.  No LDS on the way in: activations come from L2.
 // A block is four waves on the same 32 rows, each on a quarter of the block's k-range; they
@@ -178,7 +179,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
   }
 }
 
-// The same product for 33..64 tokens, where the activations are as many bytes as a block's
+// The same product for 33..128 tokens, where the activations are as many bytes as a block's
 // weights: the four waves of a block take 16 weight rows each over the block's whole k-range
 // and share one activation tile per k step through LDS (loaded once per block, not once per
 // wave).  A block is alone on its compute unit, so every wave keeps DEPTH k steps of loads
@@ -371,7 +372,7 @@ extern "C" int pi_gemm_skinny_rows_per_block(int M) { return M > SHARED_FROM_TOK
 // *splits_out tells how many splits were made (no empty ones).
 extern "C" int pi_gemm_skinny(void* C, int epilogue, long ldc, const void* X, long ldx, const void* W, long ldw, int M,
                               int N, int K, int splits, void* part, long part_elems, int* splits_out, hipStream_t stream) {
-  PI_REQUIRE(M > 0 && M <= 64 && N > 0 && K > 0, "gemm_skinny: takes 1..64 rows, got M=%d N=%d K=%d", M, N, K);
+  PI_REQUIRE(M > 0 && M <= 128 && N > 0 && K > 0, "gemm_skinny: takes 1..128 rows, got M=%d N=%d K=%d", M, N, K);
   PI_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "gemm_skinny: K (%d) and row strides (%ld, %ld) must be multiples of 8", K, ldx, ldw);
   PI_REQUIRE(((uintptr_t)X % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_skinny: operands must be 16-byte aligned");
   PI_REQUIRE(splits >= 1 && splits <= 65535, "gemm_skinny: bad split count %d", splits);
@@ -386,9 +387,14 @@ extern "C" int pi_gemm_skinny(void* C, int epilogue, long ldc, const void* X, lo
   const dim3 grid(groups, splits);
   const int mb = (M + 15) / 16;
   const bf16_t *x = (const bf16_t*)X, *w = (const bf16_t*)W;
-  if (M > SHARED_FROM_TOKENS)
-    return mb == 3 ? launch_shared<3>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part)
-                   : launch_shared<4>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
+  if (M > SHARED_FROM_TOKENS) {
+#define SHARED(B) case B: return launch_shared<B>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part)
+    switch (mb) {
+      SHARED(3); SHARED(4); SHARED(5); SHARED(6); SHARED(7);
+      default: return launch_shared<8>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
+    }
+#undef SHARED
+  }
   switch (mb) {
     case 1: return launch_mb<1>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
     case 2: return launch_mb<2>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);

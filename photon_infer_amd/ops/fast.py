@@ -23,7 +23,7 @@ import torch
 from . import _lib
 
 EPI_BF16, EPI_F32, EPI_ACCUM, EPI_SWIGLU = 0, 1, 2, 3
-SKINNY_MAX_ROWS = 64
+SKINNY_MAX_ROWS = 128          # up to this many tokens the weight-streaming kernels serve a product (measured against the tile kernel)
 ROWS_PER_BLOCK = 32            # weight rows per block of the skinny kernel
 TARGET_BLOCKS = 512            # blocks wanted in flight to keep HBM busy
 SHARED_FROM_TOKENS = 32        # more tokens than this: the skinny kernel that shares activations per block ...
@@ -31,6 +31,7 @@ SHARED_ROWS_PER_BLOCK = 64     # ... with this many weight rows per block ...
 SHARED_TARGET_BLOCKS = 256     # ... and this many blocks wanted (one per compute unit)
 GEMM_PART_FLOATS = 16 << 20    # workspace for the pieces of products split over k (64 MB)
 TILE_MAX_SPLITS = 4
+PIECES_BELOW_TILES = 200       # fewer 128 x 128 tiles than this: q, k, v of a prompt portion are left in k pieces too
 ATTN_PART_FLOATS = 4 << 20     # key-split partial results of decode attention
 MAX_DECODE_SPLITS = 64         # the combine kernel holds one key range per lane
 DECODE_WAVES_WANTED = 512      # waves of the decode attention kernel that fill the chip (measured at batch 1 to 64: more is never faster)
@@ -166,8 +167,21 @@ def gemm_pieces(a, w) -> Optional[Partials]:
     M, K = a.shape
     N = w.shape[0]
     lda, ldw = a.stride(0) if M > 1 else K, w.stride(0)
-    if M > SKINNY_MAX_ROWS or not _gemm_ok(a, w, K, lda, ldw) or a.stride(1) != 1 or w.stride(1) != 1:
+    if not _gemm_ok(a, w, K, lda, ldw) or a.stride(1) != 1 or w.stride(1) != 1:
         return None
+    if M > SKINNY_MAX_ROWS:
+        # a prompt portion of a few hundred tokens has too few 128 x 128 tiles for the chip:
+        # split k there too, the consumer adds the pieces
+        tiles = -(-M // 128) * -(-N // 128)
+        splits = _tile_splits(M, N, K) if tiles < PIECES_BELOW_TILES else 1
+        if splits <= 1:
+            return None
+        ws = workspace(a.device)
+        _flush_pending()
+        made = _lib.load("bf16").pi_gemm_mfma_pieces(K, splits)
+        _lib.call("bf16", "pi_gemm_mfma", ws.gemm_part.data_ptr(), EPI_F32, N, a.data_ptr(), lda, w.data_ptr(), ldw,
+                  M, N, K, splits, _stream())
+        return Partials(ws.gemm_part, made, M, N) if made > 1 else None
     splits = _skinny_splits(M, N, K)
     if splits <= 1:
         return None
