@@ -191,6 +191,13 @@ class ModelRunner:
         self.cache.commit_step(slots, [len(e.tokens) for e in entries])
         return logits
 
+    graphs_captured = 0
+
+    def capture_stream(self):
+        if getattr(self, "_capture_stream", None) is None:
+            self._capture_stream = torch.cuda.Stream(device=self.device)
+        return self._capture_stream
+
     def graph_pool(self):
         if getattr(self, "_graph_pool", None) is None:
             self._graph_pool = torch.cuda.graph_pool_handle()
@@ -323,25 +330,42 @@ class _DecodeGraph:
     def run(self, entries, slots, lengths, temperatures, uniforms, feed=None) -> torch.Tensor:
         self._fill(entries, slots, lengths, temperatures, uniforms, feed)
         if self.graph is None:
-            # the first step of this batch size runs eagerly (and does this step's work); the
-            # capture that follows records the same launches without running them
-            self._body()
-            torch.cuda.synchronize()
+            runner = self.runner
+            # The runner's very first decode step runs eagerly, so that everything made at first
+            # use (workspaces, kernel libraries) exists before any capture; it does the step's
+            # work, and the capture that follows only records.  Every later graph is captured
+            # straight away and replayed for its first step.
+            eager_first = not runner.graphs_captured
+            if eager_first:
+                self._body()
+                torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             # no garbage collection while the stream is capturing: a collected tensor of some
             # earlier engine (pinned memory, events) would make calls that a capture forbids
             collecting = gc.isenabled()
             gc.disable()
             try:
-                # all graphs of a runner take their intermediate buffers from one pool: they
-                # never run at the same time and hold nothing in it between replays (the
-                # sampled tokens and the metadata lie outside)
-                with torch.cuda.graph(graph, pool=self.runner.graph_pool()):
-                    self._body()
+                # Capture on a stream of the runner's own (default priority), begun and ended by
+                # hand: no device-wide wait, collection or cache flush per graph.  All graphs
+                # of a runner take their intermediate buffers from one pool: they never run at
+                # the same time and hold nothing in it between replays (the sampled tokens and
+                # the metadata lie outside).
+                side, main = runner.capture_stream(), torch.cuda.current_stream()
+                side.wait_stream(main)
+                with torch.cuda.stream(side):
+                    graph.capture_begin(pool=runner.graph_pool())
+                    try:
+                        self._body()
+                    finally:
+                        graph.capture_end()
+                main.wait_stream(side)
             finally:
                 if collecting:
                     gc.enable()
             self.graph = graph
+            runner.graphs_captured += 1
+            if not eager_first:
+                graph.replay()
         else:
             self.graph.replay()
         return self.sampled
