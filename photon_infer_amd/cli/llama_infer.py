@@ -46,7 +46,7 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--num-blocks", type=int, default=None)
     ap.add_argument("--max-batch", type=int, default=32)
     ap.add_argument("--max-step-tokens", type=int, default=2048)
-    ap.add_argument("--chunk-size", type=int, default=256)
+    ap.add_argument("--chunk-size", type=int, default=512)
     ap.add_argument("--max-model-len", type=int, default=None)
     ap.add_argument("--ignore-eos", action="store_true")
     ap.add_argument("--no-quantize", action="store_true", help="accepted and ignored: weights are never quantised")

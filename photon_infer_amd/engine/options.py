@@ -36,7 +36,8 @@ class EngineOptions:
     max_cache_tokens: Optional[int] = None  # tokens the page pool holds; None: max_batch * max_model_len
     max_batch: int = 32                  # most live requests (= state slots)
     max_step_tokens: int = 2048          # token budget of one step
-    chunk_size: int = 256                # largest prompt portion of one request in one step
+    chunk_size: int = 512                # largest prompt portion of one request in one step (the reference: 256; here a
+                                         # step of 512 tokens costs little more than one of 256)
     max_model_len: Optional[int] = None  # longest sequence; None: the model's max positions
     seed: int = 0
     device: str = "cuda:0"
