@@ -80,10 +80,13 @@ template <int HD>
 __global__ __launch_bounds__(64) void attention_combine_kernel(bf16_t* __restrict__ out, long out_stride,
                                                                const int* __restrict__ q_start,
                                                                const int* __restrict__ req_ids,
+                                                               const int* __restrict__ rows,
                                                                const float* __restrict__ part, int nh, int splits) {
   const int lane = threadIdx.x;
   const int head = blockIdx.x;
+  // where the result goes: the token row of request r (decode), or a listed row (cut tiles)
   const int r = req_ids ? req_ids[blockIdx.y] : (int)blockIdx.y;
+  const long out_row = rows ? rows[blockIdx.y] : q_start[r];
   const int rec = HD + 4;
   const float* base = part + ((long)blockIdx.y * nh + head) * splits * rec;
   // lane s holds range s (splits <= 64): maxima, weights and the total in parallel
@@ -114,7 +117,7 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(bf16_t* __restric
     }
   }
   const float inv = 1.0f / l_tot;
-  bf16_t* o = out + (long)q_start[r] * out_stride + (long)head * HD;
+  bf16_t* o = out + out_row * out_stride + (long)head * HD;
 #pragma unroll
   for (int i = 0; i < HD / 64; ++i) o[lane + i * 64] = from_float<bf16_t>(acc[i] * inv);
 }
@@ -144,10 +147,26 @@ extern "C" int pi_attention_decode(void* out, long out_stride, const void* q, lo
   if (splits > 1) {
     const dim3 cgrid(nh, R);
     if (hd == 64)
-      hipLaunchKernelGGL(attention_combine_kernel<64>, cgrid, block, 0, stream, (bf16_t*)out, out_stride, q_start, req_ids, (const float*)part, nh, splits);
+      hipLaunchKernelGGL(attention_combine_kernel<64>, cgrid, block, 0, stream, (bf16_t*)out, out_stride, q_start, req_ids, (const int*)nullptr, (const float*)part, nh, splits);
     else
-      hipLaunchKernelGGL(attention_combine_kernel<128>, cgrid, block, 0, stream, (bf16_t*)out, out_stride, q_start, req_ids, (const float*)part, nh, splits);
+      hipLaunchKernelGGL(attention_combine_kernel<128>, cgrid, block, 0, stream, (bf16_t*)out, out_stride, q_start, req_ids, (const int*)nullptr, (const float*)part, nh, splits);
     return pi_check_launch("attention_combine");
   }
   return 0;
+}
+
+// Merge partial results that the tile kernel wrote for `Z` tokens whose tiles' keys were cut in
+// `cuts` shares: part [Z, nh, cuts, hd + 4]; token z's result goes to row rows[z] of out.
+extern "C" int pi_attention_combine_rows(void* out, long out_stride, const int* rows, int Z, const void* part, int nh, int hd,
+                                         int cuts, hipStream_t stream) {
+  PI_REQUIRE(Z > 0 && Z <= 65535 && nh > 0 && cuts >= 2 && cuts <= 64 && rows && part, "attention_combine_rows: bad arguments (%d tokens, %d heads, %d cuts)", Z, nh, cuts);
+  PI_REQUIRE(hd == 64 || hd == 128, "attention_combine_rows: head_dim %d is not 64 or 128", hd);
+  const dim3 grid(nh, Z), block(64);
+  if (hd == 64)
+    hipLaunchKernelGGL(attention_combine_kernel<64>, grid, block, 0, stream, (bf16_t*)out, out_stride, (const int*)nullptr,
+                       (const int*)nullptr, rows, (const float*)part, nh, cuts);
+  else
+    hipLaunchKernelGGL(attention_combine_kernel<128>, grid, block, 0, stream, (bf16_t*)out, out_stride, (const int*)nullptr,
+                       (const int*)nullptr, rows, (const float*)part, nh, cuts);
+  return pi_check_launch("attention_combine_rows");
 }

@@ -22,7 +22,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
     bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q, long q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table,
     int table_width, const int* __restrict__ q_start, const int* __restrict__ kv_len_of,
-    const int* __restrict__ tile_req, const int* __restrict__ tile_q0, const int* __restrict__ order, int rounds, int nh,
+    const int* __restrict__ tile_req, const int* __restrict__ tile_q0, const int* __restrict__ tile_cut,
+    const int* __restrict__ tile_z0, float* __restrict__ part, const int* __restrict__ order, int rounds, int nh,
     int nkv, int page_size, float scale, int window, long num_pages_l, int TQ) {
   constexpr int F = HD / 8;                       // 16-byte operand fragments per lane and 32 keys: keys HD/16, values HD/16
   extern __shared__ __attribute__((aligned(16))) u32x4_t staged[];   // [2 buffers][4 chunks][F][64 lanes]
@@ -50,8 +51,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
     const int n_tok = min(TQ, q_len - q0);
     const int pos0 = kv_len - q_len + q0;          // position of the tile's first token
     auto first_key = [&](int pos) { return (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0; };
-    // keys the block walks
-    const int sc0 = first_key(pos0) / KEYS_PER_ROUND, sc1 = (pos0 + n_tok - 1) / KEYS_PER_ROUND + 1;
+    // keys the block walks: the tile's, or one of `cuts` equal shares of them in rounds of 128
+    // (the host cuts the key range of tiles when a step has too few tiles for the chip; the
+    // shares' results are merged by the combine kernel, as for decode attention)
+    const int cut = tile_cut[tile] & 0xff, cuts = tile_cut[tile] >> 8;
+    const int all0 = first_key(pos0) / KEYS_PER_ROUND, all1 = (pos0 + n_tok - 1) / KEYS_PER_ROUND + 1;
+    const int share = (all1 - all0 + cuts - 1) / cuts;
+    const int sc0 = all0 + cut * share, sc1 = min(all1, sc0 + share);   // may be empty: nothing seen, m stays -inf
     // tokens of this wave's columns, and the keys all / any of them see
     const int tok_a = (wave * CB * 16) / G, tok_b = min(((wave + 1) * CB * 16 - 1) / G, n_tok - 1);
     const bool active = tok_a < n_tok;
@@ -125,6 +131,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
     }
     attn_finish(st);
 
+    if (cuts > 1) {
+      // partial result [token of the cut tiles, head, cut, HD + 4] float32: O^T un-normalised, m, l
+      const int rec = HD + 4;
+      const float to_log2 = scale * PI_LOG2E;
+#pragma unroll
+      for (int c = 0; c < CB; ++c) {
+        if (!valid[c]) continue;
+        const int tok = ((wave * CB + c) * 16 + lr) / G;
+        float* mine = part + (((long)(tile_z0[tile] + tok) * nh + heads[c]) * cuts + cut) * rec;
+#pragma unroll
+        for (int db = 0; db < HD / 16; ++db) *reinterpret_cast<f32x4_t*>(mine + db * 16 + lg * 4) = st.o[db][c];
+        if (lg == 0) {
+          mine[HD] = st.m[c] * to_log2;        // base-2 scale; -inf stays -inf
+          mine[HD + 1] = st.l[c];
+        }
+      }
+      continue;
+    }
 #pragma unroll
     for (int c = 0; c < CB; ++c) {
       if (!valid[c]) continue;
@@ -152,12 +176,15 @@ extern "C" int pi_attention_tile_rows(int nh, int nkv, int hd) {
 static size_t tiles_lds_bytes(int hd) { return (size_t)2 * 4 * (hd / 8) * 64 * 16; }
 
 // `order`: [rounds, seats] tile indices (-1: none), the host's deal of the tiles to `seats`
-// blocks per kv head.
+// blocks per kv head.  tile_cut[t] = cut | cuts << 8: which of how many shares of its keys entry
+// t walks; entries with cuts > 1 write partial results for token tile_z0[t] + i to `part`
+// ([tokens, heads, cuts, hd + 4] float32), which pi_attention_combine_rows merges.
 extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void* q, long q_stride, const void* k_cache,
                                          const void* v_cache, const int* block_table, int table_width, const int* q_start,
-                                         const int* kv_len, const int* tile_req, const int* tile_q0, const int* order,
-                                         int rounds, int seats, int nh, int nkv, int hd, int page_size, float scale,
-                                         int window, long num_pages, hipStream_t stream) {
+                                         const int* kv_len, const int* tile_req, const int* tile_q0, const int* tile_cut,
+                                         const int* tile_z0, void* part, const int* order, int rounds, int seats, int nh,
+                                         int nkv, int hd, int page_size, float scale, int window, long num_pages,
+                                         hipStream_t stream) {
   PI_REQUIRE(rounds > 0 && seats > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad sizes rounds=%d seats=%d heads=%d kv_heads=%d", rounds, seats, nh, nkv);
   PI_REQUIRE(hd == 64 || hd == 128, "attention_prefill: head_dim %d is not 64 or 128", hd);
   PI_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_prefill: page size %d must be a multiple of 16", page_size);
@@ -178,7 +205,8 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
   const dim3 grid(seats, nkv), block(256);
 #define GO(H, C) hipLaunchKernelGGL((attention_tiles_kernel<H, C>), grid, block, lds, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, \
                                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, \
-                                    kv_len, tile_req, tile_q0, order, rounds, nh, nkv, page_size, scale, window, num_pages, TQ)
+                                    kv_len, tile_req, tile_q0, tile_cut, tile_z0, (float*)part, order, rounds, nh, nkv, page_size, scale, \
+                                    window, num_pages, TQ)
   if (hd == 64) GO(64, 2); else GO(128, 2);
 #undef GO
   return pi_check_launch("attention_prefill_mfma");

@@ -47,7 +47,14 @@ class _Workspace:
     def __init__(self, device):
         self.gemm_part = torch.empty(GEMM_PART_FLOATS, dtype=torch.float32, device=device)
         self.attn_part = torch.empty(ATTN_PART_FLOATS, dtype=torch.float32, device=device)
+        self.tile_part = torch.empty(4, dtype=torch.float32, device=device)   # partial results of cut tiles, grown on demand
+        self.device = device
         self.splits_out = ctypes.c_int(0)
+
+    def tile_part_for(self, floats: int) -> torch.Tensor:
+        if self.tile_part.numel() < floats:
+            self.tile_part = torch.empty(floats, dtype=torch.float32, device=self.device)
+        return self.tile_part
 
 
 @dataclass
@@ -236,26 +243,59 @@ def _tiles(ctx, tile_rows: int, window: int, num_kv_heads: int, device, skip=())
     key = (tile_rows, window, num_kv_heads, bool(skip))
     hit = cache.get(key)
     if hit is None:
-        req, q0, walks = [], [], []
+        req, q0, walks, first_row, n_tok = [], [], [], [], []
         skipped = set(skip)
+        row0 = 0
         for r, (n, kv) in enumerate(zip(ctx.q_lens, ctx.kv_lens)):
-            if r in skipped:
-                continue
-            for start in range(0, n, tile_rows):
-                req.append(r)
-                q0.append(start)
-                first = kv - n + start                         # position of the tile's first token
-                last = first + min(tile_rows, n - start) - 1
-                lo = max(0, first - window + 1) if window > 0 else 0
-                walks.append(last // 128 - lo // 128 + 1)
+            if r not in skipped:
+                for start in range(0, n, tile_rows):
+                    req.append(r)
+                    q0.append(start)
+                    first = kv - n + start                         # position of the tile's first token
+                    last = first + min(tile_rows, n - start) - 1
+                    lo = max(0, first - window + 1) if window > 0 else 0
+                    walks.append(last // 128 - lo // 128 + 1)
+                    first_row.append(row0 + start)
+                    n_tok.append(min(tile_rows, n - start))
+            row0 += n
         units = torch.cuda.get_device_properties(device).multi_processor_count
-        seats = max(1, min(len(req), ATTENTION_BLOCKS_PER_UNIT * units // max(1, num_kv_heads)))
-        order = deal_tiles(walks, seats)
-        host = np.concatenate([np.asarray(req, np.int32), np.asarray(q0, np.int32), order.reshape(-1)])
+        seats_wanted = max(1, ATTENTION_BLOCKS_PER_UNIT * units // max(1, num_kv_heads))
+        # too few tiles for the chip (a portion of a few hundred tokens): cut the key range of
+        # the long ones into equal shares; the shares' partial results are merged afterwards
+        cuts = cut_count(walks, seats_wanted)
+        t_req, t_q0, t_cut, t_z0, t_walk, rows = [], [], [], [], [], []
+        for i in range(len(req)):
+            k = cuts if cuts > 1 and walks[i] >= 2 * cuts else 1
+            z0 = len(rows) if k > 1 else 0
+            if k > 1:
+                rows.extend(range(first_row[i], first_row[i] + n_tok[i]))
+            for c in range(k):
+                t_req.append(req[i]); t_q0.append(q0[i]); t_cut.append(c | (k << 8)); t_z0.append(z0)
+                t_walk.append(-(-walks[i] // k))
+        seats = max(1, min(len(t_req), seats_wanted))
+        order = deal_tiles(t_walk, seats)
+        n = len(t_req)
+        host = np.concatenate([np.asarray(t_req, np.int32), np.asarray(t_q0, np.int32), np.asarray(t_cut, np.int32),
+                               np.asarray(t_z0, np.int32), np.asarray(rows, np.int32), order.reshape(-1)])
         dev = torch.from_numpy(host).to(device)
-        n = len(req)
-        hit = cache[key] = (dev[:n], dev[n:2 * n], dev[2 * n:], order.shape[0], seats)
+        z = len(rows)
+        hit = cache[key] = (dev[:n], dev[n:2 * n], dev[2 * n:3 * n], dev[3 * n:4 * n], dev[4 * n:4 * n + z], z,
+                            cuts if z else 1, dev[4 * n + z:], order.shape[0], seats)
     return hit
+
+
+MAX_TILE_CUTS = 8
+
+
+def cut_count(walks: List[int], seats_wanted: int) -> int:
+    """In how many shares the key range of a step's long tiles is cut: 1 unless the tiles are
+    fewer than half the blocks the chip holds; then as many as fill it, while every share keeps
+    at least two rounds of 128 keys."""
+    tiles = len(walks)
+    if tiles == 0 or tiles * 2 > seats_wanted:
+        return 1
+    cuts = min(MAX_TILE_CUTS, seats_wanted // tiles, max(walks) // 2)
+    return max(1, cuts)
 
 
 def _single_tokens(ctx, device):
@@ -321,11 +361,17 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
     singles, single_ids = _single_tokens(ctx, q.device) if G <= 16 else ((), None)
     if singles:
         decode_kernel(len(singles), single_ids.data_ptr(), max(ctx.kv_lens[r] for r in singles))
-    tile_req, tile_q0, order, rounds, seats = _tiles(ctx, tile_rows, int(window), num_kv_heads, q.device, skip=singles)
+    tile_req, tile_q0, tile_cut, tile_z0, rows, z, cuts, order, rounds, seats = _tiles(
+        ctx, tile_rows, int(window), num_kv_heads, q.device, skip=singles)
+    tile_part = workspace(q.device).tile_part_for(z * num_heads * cuts * (head_dim + 4))
     _lib.call("bf16", "pi_attention_prefill_mfma", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
               k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
-              ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(), order.data_ptr(),
-              rounds, seats, num_heads, num_kv_heads, head_dim, page_size, float(scale), int(window), pages, _stream())
+              ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(), tile_cut.data_ptr(),
+              tile_z0.data_ptr(), tile_part.data_ptr(), order.data_ptr(), rounds, seats, num_heads, num_kv_heads, head_dim,
+              page_size, float(scale), int(window), pages, _stream())
+    if z:
+        _lib.call("bf16", "pi_attention_combine_rows", out.data_ptr(), out.stride(0), rows.data_ptr(), z,
+                  tile_part.data_ptr(), num_heads, head_dim, cuts, _stream())
     return True
 
 

@@ -313,9 +313,9 @@ def dense_attention(qs, kvs, q_lens, kv_lens, scale, window):
     """Plain attention per request: the queries are the last q_len positions of kv_len keys."""
     outs = []
     for q, (k, v), n, kv in zip(qs, kvs, q_lens, kv_lens):
-        full_q = torch.zeros(kv, q.shape[1], q.shape[2])
-        full_q[kv - n:] = q
-        outs.append(P.attention(full_q, k, v, scale, window=window)[kv - n:])
+        full_q = torch.zeros(kv, q.shape[1], q.shape[2], dtype=torch.float64)   # in double: only the kernel's rounding counts
+        full_q[kv - n:] = q.double()
+        outs.append(P.attention(full_q, k.double(), v.double(), scale, window=window)[kv - n:])
     return torch.cat(outs)
 
 
@@ -340,6 +340,9 @@ ATTN_CASES = [
     (32, 1, 64, 16, [1, 70], [75, 70], None),                        # more heads per kv head than a wave's columns
     (8, 2, 128, 16, [1, 70, 1, 1, 2], [900, 300, 33, 1, 50], None),  # single tokens beside portions: two kernels share the step
     (4, 2, 64, 16, [1, 3, 1], [700, 40, 18], 25),                    # the same with a window
+    (8, 2, 64, 16, [70, 5], [2100, 40], None),                       # few tiles, many keys: their key ranges are cut and merged
+    (4, 1, 128, 16, [33, 1, 40], [1500, 900, 2100], None),           # the same at head size 128, beside a single token
+    (8, 2, 64, 32, [50], [2300], 700),                               # cut tiles with a window
 ]
 
 
@@ -378,7 +381,9 @@ def test_attention_finds_one_far_key_among_hundreds(_ops, dtype, fast):
     for kv_len, q_len, hot in [(777, 1, 3), (777, 1, 776), (640, 1, 639), (777, 1, 512), (500, 37, 15), (500, 37, 463),
                                (129, 2, 127),
                                # one long request: the decode kernel cuts it into its largest number of key ranges
-                               (9000, 1, 5), (9000, 1, 4417), (9000, 1, 8999)]:
+                               (9000, 1, 5), (9000, 1, 4417), (9000, 1, 8999),
+                               # a portion at the end of a long context: its tiles' key ranges are cut
+                               (2600, 37, 3), (2600, 37, 1290), (2600, 37, 2580)]:
         k = torch.randn(kv_len, nkv, hd, generator=g) * 0.1
         v = torch.randn(kv_len, nkv, hd, generator=g)
         q = torch.randn(q_len, nh, hd, generator=g) * 0.1

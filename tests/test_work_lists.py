@@ -4,7 +4,7 @@ import random
 import numpy as np
 import pytest
 
-from photon_infer_amd.ops.fast import deal_tiles, decode_length_bucket, decode_splits
+from photon_infer_amd.ops.fast import MAX_TILE_CUTS, cut_count, deal_tiles, decode_length_bucket, decode_splits
 
 
 @pytest.mark.parametrize("seed", range(5))
@@ -41,3 +41,12 @@ def test_decode_splits_fill_the_chip_but_respect_short_contexts():
     # the same key ranges anywhere inside a length bucket: eager steps and graph replays agree
     assert decode_length_bucket(129) == decode_length_bucket(256) == 256
     assert decode_splits(4, 8, 1025) == decode_splits(4, 8, 2048)
+
+
+def test_key_ranges_of_tiles_are_cut_only_when_the_tiles_are_few():
+    assert cut_count([], 64) == 1
+    assert cut_count([20] * 64, 64) == 1 and cut_count([20] * 33, 64) == 1      # enough tiles: none is cut
+    assert cut_count([64] * 16, 64) == 4                                        # 16 tiles, 64 blocks wanted
+    assert cut_count([64] * 2, 64) == MAX_TILE_CUTS
+    assert cut_count([5] * 16, 64) == 2                                         # a share keeps two rounds at least
+    assert cut_count([1] * 4, 64) == 1
