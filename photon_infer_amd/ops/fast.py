@@ -279,9 +279,27 @@ def _tiles(ctx, tile_rows: int, window: int, num_kv_heads: int, device, skip=())
                                np.asarray(t_z0, np.int32), np.asarray(rows, np.int32), order.reshape(-1)])
         dev = torch.from_numpy(host).to(device)
         z = len(rows)
-        hit = cache[key] = (dev[:n], dev[n:2 * n], dev[2 * n:3 * n], dev[3 * n:4 * n], dev[4 * n:4 * n + z], z,
-                            cuts if z else 1, dev[4 * n + z:], order.shape[0], seats)
+        hit = cache[key] = TilePlan(req=dev[:n], q0=dev[n:2 * n], cut=dev[2 * n:3 * n], z0=dev[3 * n:4 * n],
+                                    rows=dev[4 * n:4 * n + z], cut_tokens=z, cuts=cuts if z else 1, order=dev[4 * n + z:],
+                                    rounds=order.shape[0], seats=seats)
     return hit
+
+
+@dataclass
+class TilePlan:
+    """A step's work list for the tile kernel (device int32 arrays, one entry per tile or per
+    share of a cut tile)."""
+
+    req: torch.Tensor          # the entry's request
+    q0: torch.Tensor           # its first token among the request's tokens of this step
+    cut: torch.Tensor          # share | shares << 8 of the tile's key range
+    z0: torch.Tensor           # first row of the tile in ``rows`` (cut tiles only)
+    rows: torch.Tensor         # token rows of the cut tiles, in the order of their partial results
+    cut_tokens: int
+    cuts: int                  # shares per cut tile (the same for all of a step)
+    order: torch.Tensor        # [rounds, seats]: which entry a block takes in which round (-1: none)
+    rounds: int
+    seats: int
 
 
 MAX_TILE_CUTS = 8
@@ -361,17 +379,16 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
     singles, single_ids = _single_tokens(ctx, q.device) if G <= 16 else ((), None)
     if singles:
         decode_kernel(len(singles), single_ids.data_ptr(), max(ctx.kv_lens[r] for r in singles))
-    tile_req, tile_q0, tile_cut, tile_z0, rows, z, cuts, order, rounds, seats = _tiles(
-        ctx, tile_rows, int(window), num_kv_heads, q.device, skip=singles)
-    tile_part = workspace(q.device).tile_part_for(z * num_heads * cuts * (head_dim + 4))
+    plan = _tiles(ctx, tile_rows, int(window), num_kv_heads, q.device, skip=singles)
+    tile_part = workspace(q.device).tile_part_for(plan.cut_tokens * num_heads * plan.cuts * (head_dim + 4))
     _lib.call("bf16", "pi_attention_prefill_mfma", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
               k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
-              ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), tile_req.data_ptr(), tile_q0.data_ptr(), tile_cut.data_ptr(),
-              tile_z0.data_ptr(), tile_part.data_ptr(), order.data_ptr(), rounds, seats, num_heads, num_kv_heads, head_dim,
-              page_size, float(scale), int(window), pages, _stream())
-    if z:
-        _lib.call("bf16", "pi_attention_combine_rows", out.data_ptr(), out.stride(0), rows.data_ptr(), z,
-                  tile_part.data_ptr(), num_heads, head_dim, cuts, _stream())
+              ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), plan.req.data_ptr(), plan.q0.data_ptr(), plan.cut.data_ptr(),
+              plan.z0.data_ptr(), tile_part.data_ptr(), plan.order.data_ptr(), plan.rounds, plan.seats, num_heads,
+              num_kv_heads, head_dim, page_size, float(scale), int(window), pages, _stream())
+    if plan.cut_tokens:
+        _lib.call("bf16", "pi_attention_combine_rows", out.data_ptr(), out.stride(0), plan.rows.data_ptr(), plan.cut_tokens,
+                  tile_part.data_ptr(), num_heads, head_dim, plan.cuts, _stream())
     return True
 
 
