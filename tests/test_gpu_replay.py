@@ -173,6 +173,28 @@ def test_long_decoding(model_dirs, tmp_path, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_late_portions_of_a_long_prompt(model_dirs, tmp_path, dtype, monkeypatch):
+    """Short portions near the end of the longest context the model allows, beside a second
+    request's single tokens: in bfloat16 the portions' few tiles have their key ranges cut
+    into shares, and the single tokens go to the key-split kernel in the same step."""
+    reqs = requests_for("D", [500, 130], seed=6)
+    a = cut_steps("r0", reqs["r0"], [440, 40, 3, 17])
+    b = cut_steps("r1", reqs["r1"], [127, 1, 1, 1])
+    steps = [b[0], a[0]]
+    for i in range(1, 4):                                   # steps that hold a late portion of r0 and one token of r1
+        steps.append({"entries": a[i]["entries"] + b[i]["entries"], "end": a[i]["end"] + b[i]["end"]})
+    for i, st in enumerate(steps):
+        st["step"] = i
+    from photon_infer_amd.ops import fast
+    cuts_made, count = [], fast.cut_count
+    monkeypatch.setattr(fast, "cut_count", lambda walks, seats: cuts_made.append(count(walks, seats)) or cuts_made[-1])
+    runner = runner_for(model_dirs["D"], "D", dtype, live_token_need(steps))
+    check(run_trace(runner, steps, str(tmp_path)), model_dirs["D"], reqs, dtype, "late portions")
+    if dtype == "bfloat16":
+        assert max(cuts_made) > 1, "no tile's key range was cut: the test does not reach what it is for"
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", MODELS)
 def test_first_tokens_of_a_sequence(model_dirs, tmp_path, name, dtype):
     reqs = requests_for(name, [4, 4, 4], seed=5)
