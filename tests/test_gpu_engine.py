@@ -265,3 +265,38 @@ def test_cpp_program_generates_what_the_python_entry_point_generates(model_dirs,
     assert r.returncode == 0, (r.stdout, r.stderr)
     got = [[int(t) for t in line.split()] for line in r.stdout.strip().splitlines()]
     assert got == want
+
+
+@pytest.mark.parametrize("name,dtype", [("A", "float32"), ("D", "bfloat16")])
+def test_random_workloads_do_not_depend_on_graphs_or_on_running_ahead(tmp_path, name, dtype):
+    """Seeded random workloads (prompt and output lengths, temperatures, arrival steps, pool
+    and batch sizes small enough to force preemption): the tokens and the reasons for ending
+    are the same with and without graphs, with and without the step ahead, and no page or
+    slot is lost."""
+    import random
+
+    d = make_model_dir(tmp_path, name, seed=41)
+    vocab, block = ALL[name][0]["vocab_size"], ALL[name][1]["block_size"]
+    for seed in range(4):
+        rng = random.Random(1000 * seed + len(name))
+        n = rng.randint(3, 8)
+        reqs = [(random_tokens(rng.randint(1, 50), vocab, 100 * seed + i), rng.randint(1, 20), rng.choice([0.0, 0.0, 0.7, 1.1]),
+                 rng.randint(0, 25)) for i in range(n)]
+        opts = dict(num_blocks=rng.choice([12, 20, 40, 128]), max_batch=rng.choice([2, 3, 4, 6]), chunk_size=rng.choice([4, 8, 16]),
+                    max_step_tokens=rng.choice([8, 16, 48]))
+        outcomes = {}
+        for lookahead, graphs in ((False, False), (False, True), (True, True)):
+            eng = engine(d, name, dtype=dtype, block_size=block, lookahead=lookahead, use_graphs=graphs, **opts)
+            waiting, ids, step = sorted(range(n), key=lambda i: reqs[i][3]), {}, 0
+            while waiting or eng.has_work():
+                while waiting and reqs[waiting[0]][3] <= step:
+                    i = waiting.pop(0)
+                    ids[i] = eng.add_request(reqs[i][0], reqs[i][1], temperature=reqs[i][2], seed=seed + i, ignore_eos=seed % 2 == 0)
+                eng.step()
+                step += 1
+                assert step < 3000, "the engine makes no progress"
+            eng.runner.cache.check_invariants()
+            assert eng.runner.cache.num_live == 0
+            outcomes[(lookahead, graphs)] = [(eng.get_result(ids[i]), eng.get_request(ids[i]).finish_reason) for i in range(n)]
+        assert outcomes[(False, True)] == outcomes[(False, False)], (seed, opts)
+        assert outcomes[(True, True)] == outcomes[(False, False)], (seed, opts)
