@@ -289,7 +289,10 @@ class ContinuousBatchScheduler:
                 break
             n = min(req.remaining(), self.chunk_size, budget)
             need = self.cache.pages_needed(None, n)
-            if not self._fits(need, held):
+            # room for everything the request already brings (its prompt, and what it generated
+            # before a preemption), not only for this portion: admitting on the first portion
+            # alone lets requests in that are preempted again before their prompt is through
+            if not self._fits(self.cache.pages_needed(None, req.remaining()), held):
                 if not self.running and not batch.items:
                     # nothing else holds pages: this request can never start
                     self.waiting.popleft()

@@ -128,6 +128,26 @@ def test_out_of_pages_preempts_the_newest_and_recomputes_it():
     assert cache.free_pages() == 6 and cache.num_live == 0
 
 
+def test_a_request_waits_until_its_whole_prompt_has_room():
+    """Admission wants room for the whole prompt, not only for the first portion: a request
+    let in on less would be preempted before its prompt is through."""
+    cache, s = make(pages=8, page=4, budget=16, chunk=4)         # 32 tokens in the pool
+    a = s.add_request(list(range(20)), SamplingParams(max_new_tokens=4))
+    b1 = s.schedule_next_batch()
+    run_step(cache, s, b1)                                       # a holds one page, seven are free
+    b = s.add_request(list(range(30)), SamplingParams(max_new_tokens=2))      # 8 pages: one portion fits, the prompt does not
+    b2 = s.schedule_next_batch()
+    assert [(r.request_id, n) for r, n in b2.items] == [(a, 4)]
+    assert s.get_request(b).state is RequestState.WAITING
+    run_step(cache, s, b2)
+    while s.get_request(a).state is not RequestState.FINISHED:   # a runs to its end alone
+        batch = s.schedule_next_batch()
+        assert all(r.request_id == a for r, _ in batch.items)
+        run_step(cache, s, batch)
+    b3 = s.schedule_next_batch()                                 # now the pool is empty: b's prompt has room
+    assert [(r.request_id, n) for r, n in b3.items] == [(b, 4)]
+
+
 def test_a_request_that_cannot_fit_alone_is_finished_not_hung():
     cache, s = make(pages=2, budget=64, chunk=64)       # 8 tokens of cache
     a = s.add_request([1] * 12, SamplingParams(max_new_tokens=4))     # can never start
