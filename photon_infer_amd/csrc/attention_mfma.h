@@ -29,7 +29,8 @@ struct AttnState {
   Frag q[CB][HD / 32];
   f32x4_t o[HD / 16][CB];
   float m[CB];          // reference score of the column (raw units, see attn_compute)
-  float l[CB];          // this lane's share of the column's sum of weights: attn_finish adds the four shares
+  f32x4_t ls[CB];       // the column's sum of weights, four times over (see weight_sum)
+  float l[CB];          // the same as a scalar, set by attn_finish
   int pos[CB];          // last visible key of the column
   int lo[CB];           // first visible key of the column
 };
@@ -59,16 +60,27 @@ __device__ inline void attn_init(AttnState<HD, CB>& st) {
   for (int c = 0; c < CB; ++c) {
     st.m[c] = -INFINITY;
     st.l[c] = 0.f;
+    st.ls[c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int db = 0; db < HD / 16; ++db) st.o[db][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
   }
 }
 
-// After the last chunk: the column's sum of weights from the four lanes that share it.
+// The sum of a column's weights is left to the matrix unit: a product with sixteen value rows
+// of ones adds the 32 weights of a chunk, exactly as rounded for the product with the values,
+// and gives every lane of the column the whole sum.  The vector unit, which the weights keep
+// busy, is spared eight additions per column and chunk and the exchange between lanes.
+__device__ inline f32x4_t weight_sum(const Frag& weights, f32x4_t acc) {
+  Frag ones;
+  ones.n = u32x4_t{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  return mfma16(ones, weights, acc);
+}
+
+// After the last chunk.
 template <int HD, int CB>
 __device__ inline void attn_finish(AttnState<HD, CB>& st) {
 #pragma unroll
-  for (int c = 0; c < CB; ++c) st.l[c] = column_sum(st.l[c]);
+  for (int c = 0; c < CB; ++c) st.l[c] = st.ls[c][0];
 }
 
 // Where the two key tiles of a chunk lie: page id (-1: none) and first slot in the page.  The
@@ -188,47 +200,148 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KV& kv, int k0,
         }
         mx = fmaxf(mx, s[t][c][i]);
       }
+    // weights 2^((score - reference) * scale), summed and folded into the accumulators; a column
+    // that has seen nothing yet has only -inf scores
+    auto fold = [&](float m_ref) {
+      float mc = m_ref * scale_log2;
+      if (MASKED) mc = (m_ref == -INFINITY) ? 0.f : mc;
+      float p[2][4];
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) p[t][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][c][i], scale_log2, -mc));
+      Frag pb;
+      pb.q.x = pack_bf16x2(p[0][0], p[0][1]);
+      pb.q.y = pack_bf16x2(p[0][2], p[0][3]);
+      pb.q.z = pack_bf16x2(p[1][0], p[1][1]);
+      pb.q.w = pack_bf16x2(p[1][2], p[1][3]);
+      st.ls[c] = weight_sum(pb, st.ls[c]);
+#pragma unroll
+      for (int db = 0; db < HD / 16; ++db) {
+        Frag va = kv.val(db);
+        if (MASKED) {   // a missing tile was read from page 0: its values must not meet even a zero weight
+          if (!kv.have[0]) va.d[0] = make_uint2(0u, 0u);
+          if (!kv.have[1]) va.d[1] = make_uint2(0u, 0u);
+        }
+        st.o[db][c] = mfma16(va, pb, st.o[db][c]);
+      }
+    };
     // the cheap test first: does any lane hold a score that far above its column's reference?
-    float m_ref = st.m[c];
+    const float m_ref = st.m[c];
     if (__builtin_expect(__builtin_amdgcn_ballot_w64(mx > m_ref + slack) != 0, 0)) {   // also at the first visible key: m_ref is -inf then
       mx = column_max(mx);
       const bool move = mx > m_ref + slack;
       const float alpha = move ? __builtin_amdgcn_exp2f((m_ref - mx) * scale_log2) : 1.f;
-      m_ref = move ? mx : m_ref;
-      st.m[c] = m_ref;
-      st.l[c] *= alpha;
+      const float m_new = move ? mx : m_ref;
+      st.m[c] = m_new;
+      st.ls[c][0] *= alpha; st.ls[c][1] *= alpha; st.ls[c][2] *= alpha; st.ls[c][3] *= alpha;
+#pragma unroll
+      for (int db = 0; db < HD / 16; ++db) {
+        st.o[db][c][0] *= alpha; st.o[db][c][1] *= alpha; st.o[db][c][2] *= alpha; st.o[db][c][3] *= alpha;
+      }
+      // The fold is written out on both paths, and the marker keeps the compiler from joining
+      // them again: joined, the accumulators of the common path would be copied to where the
+      // rescaled ones lie, 16 registers per column and chunk.
+      fold(m_new);
+      asm volatile("" ::: "memory");
+    } else {
+      fold(m_ref);
+    }
+  }
+}
+
+// Fold NJ staged chunks that every column sees whole (no per-key tests, every page there).
+// `from`: this lane's first fragment of the first chunk in LDS (StagedChunk's order);
+// `chunk_stride`: 16-byte units from one chunk to the next.  All scores of the group are
+// formed first, then one test decides whether any column's reference has to move, then the
+// weights and the accumulation run as straight-line code: matrix and vector instructions of
+// different chunks and columns can overlap, and the test costs one branch per group.
+template <int HD, int CB, int NJ>
+__device__ inline void attn_compute_plain(AttnState<HD, CB>& st, const u32x4_t* from, int chunk_stride, float scale_log2) {
+  // The key fragments of a chunk are read from LDS while the products of the chunk before it
+  // run; the scheduler is told so, or it reads each fragment right before its use to save
+  // registers and the wave waits for LDS sixteen times per group.
+  constexpr int KF = 2 * (HD / 32);
+  Frag kf[2][KF];
+  f32x4_t s[NJ][2][CB];
+#pragma unroll
+  for (int f = 0; f < KF; ++f) kf[0][f].n = from[f * 64];
+#pragma unroll
+  for (int j = 0; j < NJ; ++j) {
+    if (j + 1 < NJ) {
+#pragma unroll
+      for (int f = 0; f < KF; ++f) kf[(j + 1) & 1][f].n = from[(j + 1) * chunk_stride + f * 64];
+    }
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+      for (int c = 0; c < CB; ++c) s[j][t][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < HD / 32; ++ks)
+#pragma unroll
+        for (int c = 0; c < CB; ++c) s[j][t][c] = mfma16(kf[j & 1][t * (HD / 32) + ks], st.q[c][ks], s[j][t][c]);
+    }
+    if (j + 1 < NJ) __builtin_amdgcn_sched_group_barrier(0x100, KF, 0);   // LDS reads of the next chunk
+    __builtin_amdgcn_sched_group_barrier(0x008, KF * CB, 0);               // this chunk's products
+  }
+  const float slack = PI_RESCALE_SLACK / scale_log2;
+  float mx[CB];
+  bool rise = false;
+#pragma unroll
+  for (int c = 0; c < CB; ++c) {
+    mx[c] = -INFINITY;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j)
+#pragma unroll
+      for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) mx[c] = fmaxf(mx[c], s[j][t][c][i]);
+    rise = rise || mx[c] > st.m[c] + slack;
+  }
+  auto fold = [&]() {
+    float mc[CB];
+#pragma unroll
+    for (int c = 0; c < CB; ++c) mc[c] = st.m[c] * scale_log2;
+#pragma unroll
+    for (int j = 0; j < NJ; ++j) {
+      Frag va[HD / 16];
+#pragma unroll
+      for (int db = 0; db < HD / 16; ++db) va[db].n = from[j * chunk_stride + (HD / 16 + db) * 64];
+#pragma unroll
+      for (int c = 0; c < CB; ++c) {
+        float p[2][4];
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) p[t][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j][t][c][i], scale_log2, -mc[c]));
+        Frag pb;
+        pb.q.x = pack_bf16x2(p[0][0], p[0][1]);
+        pb.q.y = pack_bf16x2(p[0][2], p[0][3]);
+        pb.q.z = pack_bf16x2(p[1][0], p[1][1]);
+        pb.q.w = pack_bf16x2(p[1][2], p[1][3]);
+      st.ls[c] = weight_sum(pb, st.ls[c]);
+#pragma unroll
+        for (int db = 0; db < HD / 16; ++db) st.o[db][c] = mfma16(va[db], pb, st.o[db][c]);
+      }
+    }
+  };
+  if (__builtin_expect(__builtin_amdgcn_ballot_w64(rise) != 0, 0)) {   // also at the first keys: the references are -inf then
+#pragma unroll
+    for (int c = 0; c < CB; ++c) {
+      const float top = column_max(mx[c]);
+      const bool move = top > st.m[c] + slack;
+      const float alpha = move ? __builtin_amdgcn_exp2f((st.m[c] - top) * scale_log2) : 1.f;
+      st.m[c] = move ? top : st.m[c];
+      st.ls[c][0] *= alpha; st.ls[c][1] *= alpha; st.ls[c][2] *= alpha; st.ls[c][3] *= alpha;
 #pragma unroll
       for (int db = 0; db < HD / 16; ++db) {
         st.o[db][c][0] *= alpha; st.o[db][c][1] *= alpha; st.o[db][c][2] *= alpha; st.o[db][c][3] *= alpha;
       }
     }
-    // weights 2^((score - reference) * scale); a column that has seen nothing yet has only -inf scores
-    float mc = m_ref * scale_log2;
-    if (MASKED) mc = (m_ref == -INFINITY) ? 0.f : mc;
-    float p[2][4];
-    float sum = 0.f;
-#pragma unroll
-    for (int t = 0; t < 2; ++t)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        p[t][i] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[t][c][i], scale_log2, -mc));
-        sum += p[t][i];
-      }
-    st.l[c] += sum;
-    Frag pb;
-    pb.q.x = pack_bf16x2(p[0][0], p[0][1]);
-    pb.q.y = pack_bf16x2(p[0][2], p[0][3]);
-    pb.q.z = pack_bf16x2(p[1][0], p[1][1]);
-    pb.q.w = pack_bf16x2(p[1][2], p[1][3]);
-#pragma unroll
-    for (int db = 0; db < HD / 16; ++db) {
-      Frag va = kv.val(db);
-      if (MASKED) {   // a missing tile was read from page 0: its values must not meet even a zero weight
-        if (!kv.have[0]) va.d[0] = make_uint2(0u, 0u);
-        if (!kv.have[1]) va.d[1] = make_uint2(0u, 0u);
-      }
-      st.o[db][c] = mfma16(va, pb, st.o[db][c]);
-    }
+    fold();                          // written out on both paths, see attn_compute
+    asm volatile("" ::: "memory");
+  } else {
+    fold();
   }
 }
 

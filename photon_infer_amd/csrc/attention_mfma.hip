@@ -16,6 +16,9 @@
 #include "attention_mfma.h"
 
 #define KEYS_PER_ROUND 128
+#ifndef PLAIN_NJ
+#define PLAIN_NJ 4   // chunks of a fully visible round that are folded as one group (2 or 4)
+#endif
 
 template <int HD, int CB>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2 : 1))) void attention_tiles_kernel(
@@ -113,7 +116,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
     for (int sc = sc0; sc < sc1; ++sc) {
       const int buf = (sc - sc0) & 1;
       fetch();                                     // the next 128 keys (past the end: no pages, page 0 is read)
-      if (active) {
+      // a round that every column of the wave sees whole, with every page there: straight-line
+      // code without the per-key tests (the accumulators then stay in place from chunk to chunk)
+      const int round0 = sc * KEYS_PER_ROUND;
+      const bool missing = __builtin_amdgcn_ballot_w64(lane < 8 && !(&present[buf][0][0])[lane % 8]) != 0;
+      if (active && !missing && round0 >= see_all_lo && round0 + KEYS_PER_ROUND - 1 <= see_all_hi) {
+        attn_compute_plain<HD, CB, PLAIN_NJ>(st, staged + (buf * 4 * F) * 64 + lane, F * 64, scale_log2);
+        if (PLAIN_NJ < 4) attn_compute_plain<HD, CB, PLAIN_NJ>(st, staged + ((buf * 4 + 2) * F) * 64 + lane, F * 64, scale_log2);
+      } else if (active) {
 #pragma unroll 1
         for (int j = 0; j < 4; ++j) {
           const int key0 = sc * KEYS_PER_ROUND + j * 32;
