@@ -354,18 +354,23 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KV& kv, int k0,
 // Walk chunks c0 .. c1-1 (32 keys each) with the next chunk's loads in flight during the
 // current chunk's arithmetic.  Chunks from `first_unmasked` up to `last_unmasked` (inclusive)
 // are known to be fully visible to every column.
-template <int HD, int CB>
+// `meanwhile` is called once the first chunk's loads are on their way (also when the range is
+// empty): work that the walk needs but the loads do not, such as fetching the queries.
+template <int HD, int CB, class Meanwhile>
 __device__ inline void attn_walk(AttnState<HD, CB>& st, int c0, int c1, int first_unmasked, int last_unmasked,
                                  const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache,
                                  const int* __restrict__ bt, int table_width, int kv_len, int nkv, int g, int page_size,
-                                 long num_pages_l, float scale_log2, int lane) {
+                                 long num_pages_l, float scale_log2, int lane, Meanwhile&& meanwhile) {
   // the range is the same in every lane; saying so keeps the loop's branches scalar, and a
   // divergent break would make the compiler wait for every load at the loop's head
   c0 = __builtin_amdgcn_readfirstlane(c0);
   c1 = __builtin_amdgcn_readfirstlane(c1);
   first_unmasked = __builtin_amdgcn_readfirstlane(first_unmasked);
   last_unmasked = __builtin_amdgcn_readfirstlane(last_unmasked);
-  if (c0 >= c1) return;
+  if (c0 >= c1) {
+    meanwhile();
+    return;
+  }
   KVChunk<HD> a, b;
   KVLaneOffsets<HD> off;
   off.set(page_size, lane);
@@ -379,6 +384,7 @@ __device__ inline void attn_walk(AttnState<HD, CB>& st, int c0, int c1, int firs
   // loaded and never used.
   ChunkPages pa = cur.next(), pb = cur.next();
   attn_load<HD>(a, pa, k_cache, v_cache, off, nkv, g, page_size, num_pages);
+  meanwhile();
   for (int c = c0; c < c1; c += 2) {
     pa = cur.next();
     attn_load<HD>(b, pb, k_cache, v_cache, off, nkv, g, page_size, num_pages);

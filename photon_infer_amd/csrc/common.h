@@ -70,6 +70,29 @@ __device__ inline float wave_max(float v) {
   return v;
 }
 
+// A rotated pair: (a, b) turned by the angle whose cosine and sine are c and s.  One spelling
+// for every kernel that rotates, with the roundings fixed, so that a query or key comes out the
+// same wherever it is rotated.
+__device__ inline void rope_pair(float a, float b, float c, float s, float& lo, float& hi) {
+  lo = __builtin_fmaf(a, c, -(b * s));
+  hi = __builtin_fmaf(a, s, b * c);
+}
+
+// Element i of a product that is still split over k: the sum of its float32 pieces
+// ([splits] planes of part_stride floats), added in split order, eight loads in flight.
+__device__ inline float split_sum(const float* __restrict__ part, int splits, long part_stride, long i) {
+  float val = 0.f;
+  const float* p = part + i;
+  for (int s0 = 0; s0 < splits; s0 += 8) {
+    float tmp[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) tmp[u] = (s0 + u < splits) ? p[(s0 + u) * part_stride] : 0.f;
+#pragma unroll
+    for (int u = 0; u < 8; ++u) val += tmp[u];
+  }
+  return val;
+}
+
 // ---- reductions over the four lanes l, l+16, l+32, l+48 (one column of a matrix-core tile),
 // with the gfx950 row / half swaps instead of a trip through the LDS crossbar:
 // v_permlane16_swap exchanges the odd 16-lane rows of one register with the even rows of the

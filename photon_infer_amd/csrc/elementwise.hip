@@ -171,16 +171,7 @@ extern "C" int pi_rope_table(float* table, const int* positions, const float* in
 template <typename T>
 __device__ inline float rope_source(const T* __restrict__ src, const float* __restrict__ part, int splits, long part_stride, int i) {
   if (!part) return to_float(src[i]);
-  float val = 0.f;
-  const float* p = part + i;
-  for (int s0 = 0; s0 < splits; s0 += 8) {      // loads go out together, adds keep the split order
-    float tmp[8];
-#pragma unroll
-    for (int u = 0; u < 8; ++u) tmp[u] = (s0 + u < splits) ? p[(s0 + u) * part_stride] : 0.f;
-#pragma unroll
-    for (int u = 0; u < 8; ++u) val += tmp[u];
-  }
-  return val;
+  return split_sum(part, splits, part_stride, i);
 }
 
 // One wave per (token, head), four heads to a block; a lane owns whole pairs, so nothing is
@@ -236,8 +227,10 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
       const float a = rope_source(src, pp, splits, part_stride, i0);
       const float b = rope_source(src, pp, splits, part_stride, i1);
       const float c = table[t * rotary_dim + j], s = table[t * rotary_dim + half + j];
-      dst[i0 * dst_stride] = from_float<T>(a * c - b * s);
-      dst[i1 * dst_stride] = from_float<T>(a * s + b * c);
+      float lo, hi;
+      rope_pair(a, b, c, s, lo, hi);
+      dst[i0 * dst_stride] = from_float<T>(lo);
+      dst[i1 * dst_stride] = from_float<T>(hi);
     }
     if (part || dst != src)
       for (int i = rotary_dim + lane; i < hd; i += PI_WAVE) dst[i * dst_stride] = from_float<T>(rope_source(src, pp, splits, part_stride, i));
@@ -297,8 +290,7 @@ __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
         for (int e = 0; e < 2; ++e) {
           const int i = 2 * w + e;
           const float cc = i < 4 ? c0[i] : c1[i - 4], ss = i < 4 ? s0[i] : s1[i - 4];
-          rl[e] = a[e] * cc - b[e] * ss;
-          rh[e] = a[e] * ss + b[e] * cc;
+          rope_pair(a[e], b[e], cc, ss, rl[e], rh[e]);
         }
         ol[w] = f32x2_to_bf16x2_bits(rl[0], rl[1]);
         oh[w] = f32x2_to_bf16x2_bits(rh[0], rh[1]);

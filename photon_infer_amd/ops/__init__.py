@@ -322,6 +322,37 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
         block_table.shape[1] if write else 0, page_size if write else 0, pages, None, 0, 0, 0, 0, 0, _stream())
 
 
+def decode_attention_from_projection(out: torch.Tensor, qkv, ctx, rotary, num_heads: int, num_kv_heads: int,
+                                     head_dim: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                                     block_table: torch.Tensor, page_size: int, scale: float, window: int,
+                                     write_kv: bool) -> bool:
+    """For a step that holds single tokens only: rotation, cache write and attention in one
+    kernel, from the q|k|v projection ``qkv`` (a tensor [T, N] or ``fast.Partials``, columns
+    [q heads | k heads | v heads]).  Returns False, having done nothing, when the step, the
+    sizes or the rotation (``rotary`` as for ``rope_kv_write``; only the whole head with paired
+    halves, or none) are not what that kernel serves; the caller then takes the separate kernels."""
+    if not (_FAST and out.dtype == torch.bfloat16 and out.is_cuda and getattr(ctx, "all_decode", False)):
+        return False
+    from . import fast
+    if not isinstance(qkv, fast.Partials) and qkv.dtype != torch.bfloat16:
+        return False
+    T = out.shape[0]
+    table = None
+    if rotary is not None:
+        src, rdim, inter = rotary
+        if rdim != head_dim or inter:
+            return False
+        _ptr_unused, _rdim, _inter, table = _rotary_args(rotary, ctx.positions, T)
+    check_attention_sizes(num_heads, num_kv_heads, head_dim)
+    if out.shape != (T, num_heads * head_dim):
+        raise KernelError(f"attention: out {tuple(out.shape)} does not match {num_heads} x {head_dim}")
+    pages = _check_cache(k_cache, v_cache, num_kv_heads, head_dim, page_size, out.dtype)
+    if block_table.dim() != 2 or block_table.dtype != torch.int32 or not block_table.is_contiguous():
+        raise KernelError("attention: block table must be contiguous int32 [requests, width]")
+    return fast.decode_attention_from_projection(out, qkv, ctx, table, num_heads, num_kv_heads, head_dim, k_cache, v_cache,
+                                                 block_table, page_size, scale, window, pages, write_kv)
+
+
 def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     block_table: torch.Tensor, ctx, num_heads: int, num_kv_heads: int, head_dim: int,
                     page_size: int, scale: float, window: int = 0) -> None:

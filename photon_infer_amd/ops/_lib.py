@@ -31,6 +31,7 @@ _SIGNATURES = {
         "pi_attention_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, L, P],
         "pi_attention_combine_rows": [P, L, P, I, P, I, I, I, P],
         "pi_attention_decode": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, L, I, P, L, P],
+        "pi_attention_decode_fused": [P, L, P, L, P, I, I, I, P, I, P, P, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, P],
     },
 }
 

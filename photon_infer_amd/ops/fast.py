@@ -392,6 +392,35 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
     return True
 
 
+def decode_attention_from_projection(out, qkv, ctx, table, num_heads, num_kv_heads, head_dim, k_cache, v_cache,
+                                     block_table, page_size, scale, window, pages, write_kv) -> bool:
+    """A step of single tokens: attention straight from the q|k|v projection (``qkv``: a bfloat16
+    tensor [T, N] or ``Partials``), which the kernel rotates by ``table`` (the step's cos / sin
+    table [T, head_dim], or None) and whose keys and values it stores.  False: not for these sizes."""
+    G = num_heads // num_kv_heads
+    if not ctx.all_decode or G > 16 or head_dim not in (64, 128) or page_size % 16 or out.stride(0) % 4:
+        return False
+    R = ctx.R
+    pieces = isinstance(qkv, Partials)
+    need = (num_heads + (2 * num_kv_heads if write_kv else 0)) * head_dim
+    if (qkv.M if pieces else qkv.shape[0]) != R or (qkv.N if pieces else qkv.shape[1]) < need:
+        return False
+    if (qkv.N % 4 or qkv.part.data_ptr() % 16) if pieces else (qkv.stride(0) % 8 or qkv.stride(1) != 1 or qkv.data_ptr() % 16):
+        return False
+    splits = decode_splits(R, num_kv_heads, ctx.max_kv_len)
+    ws = workspace(out.device)
+    while splits > 1 and R * num_heads * splits * (head_dim + 4) > ws.attn_part.numel():
+        splits -= 1
+    _lib.call("bf16", "pi_attention_decode_fused", out.data_ptr(), out.stride(0),
+              None if pieces else qkv.data_ptr(), 0 if pieces else qkv.stride(0),
+              qkv.part.data_ptr() if pieces else None, qkv.splits if pieces else 0, qkv.N if pieces else 0, R,
+              None if table is None else table.data_ptr(), int(bool(write_kv)), k_cache.data_ptr(), v_cache.data_ptr(),
+              block_table.data_ptr(), block_table.shape[1], ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), R, num_heads,
+              num_kv_heads, head_dim, page_size, float(scale), int(window), pages, splits, ws.attn_part.data_ptr(),
+              ws.attn_part.numel(), _stream())
+    return True
+
+
 def plan_attention(q_lens, kv_lens) -> dict:
     return {}
 

@@ -88,6 +88,14 @@ class PagedAttention(Mixer):
         fused_position = self.position is None or rotary is not None
         table = ctx.block_tables[cache.group]
         qkv = ops.qkv_projection(h, self.w_qkv, self.dtype) if fused_position else None
+        if qkv is not None and ctx.all_decode:
+            # single tokens only: one kernel rotates, writes the cache and attends
+            attn = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
+            if ops.decode_attention_from_projection(attn, qkv, ctx, rotary, self.num_heads, self.num_kv_heads,
+                                                    self.head_dim, cache.k, cache.v, table, cache.page_size, self.scale,
+                                                    self.window or 0, writes):
+                ops.gemm(x, attn, self.w_o, accumulate=True, may_defer=True)
+                return
         if qkv is not None and not isinstance(qkv, torch.Tensor):
             # the projection is still in pieces (split over k): the rotation kernel sums them
             q = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)

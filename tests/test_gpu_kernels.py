@@ -308,6 +308,94 @@ def test_rope_kv_write_many_tokens(_ops, hd, page, rotate):
     assert vc_h.permute(0, 1, 3, 2)[~written.unsqueeze(1).expand(-1, nkv, -1)].abs().max() == 0
 
 
+@pytest.mark.parametrize("hd,nh,nkv,page,window,rotate", [(64, 8, 2, 16, 0, True), (128, 4, 4, 32, 40, True), (64, 6, 2, 16, 24, False),
+                                                          (128, 16, 1, 16, 0, True)])
+@pytest.mark.parametrize("pieces", [False, True])
+def test_decode_attention_from_projection(_ops, hd, nh, nkv, page, window, rotate, pieces):
+    """A step of single tokens through the kernel that rotates, writes the cache and attends at
+    once: the cache it leaves and its outputs are, bit for bit, those of the separate kernels
+    (a token's logits must not depend on what else the step held), and the outputs agree with
+    plain attention over that cache.  The new token at a page's first and
+    last slot, a context of one token, few and many keys, the projection as a tensor and as
+    float32 pieces.  The slot of the new token holds large numbers beforehand: a kernel that
+    read it before it was written, or counted the token twice, or not at all, would show."""
+    from photon_infer_amd.ops import fast
+    kv_lens = [1, page, page + 1, 2 * page + 1, 300, 1000, 65]
+    R = len(kv_lens)
+    ctx = attention_ctx([1] * R, kv_lens, BF16)
+    g = gen(hd + nh + page)
+    seqs = [(torch.randn(kv, nkv, hd, generator=g) * 0.5, torch.randn(kv, nkv, hd, generator=g)) for kv in kv_lens]
+    kv = PagedKV(seqs, page, BF16, seed=3)
+    table = kv.table.cpu()
+    for r, n in enumerate(kv_lens):
+        pg, sl = table[r, (n - 1) // page].item(), (n - 1) % page
+        kv.k[pg, :, sl] = 1e4
+        kv.v[pg, :, :, sl] = -1e4
+    N = (nh + 2 * nkv) * hd
+    if pieces:
+        part = (torch.randn(3, R, N, generator=g) * 0.4).to(DEV)
+        qkv = fast.Partials(part, 3, R, N)
+    else:
+        qkv = (torch.randn(R, N, generator=g) * 0.6).to(BF16).to(DEV)
+    freqs = P.rope_frequencies(hd, 10000.0, None)
+    inv = torch.tensor(freqs, dtype=torch.float64).to(F32).to(DEV)
+    rotary = (inv, hd, False) if rotate else None
+    scale = hd ** -0.5
+
+    # the separate kernels, on a copy of the cache
+    k1, v1 = kv.k.clone(), kv.v.clone()
+    if pieces:
+        q = torch.empty(R, nh * hd, dtype=BF16, device=DEV)
+        _ops.rope_kv_write(q, None, None, ctx.positions, ctx.req_of_token, rotary, nh, nkv, hd, k1, v1, kv.table, page,
+                           pieces=qkv, write_kv=True)
+    else:
+        own = qkv.clone()
+        q = own[:, :nh * hd]
+        _ops.rope_kv_write(q, own[:, nh * hd:(nh + nkv) * hd], own[:, (nh + nkv) * hd:], ctx.positions, ctx.req_of_token,
+                           rotary, nh, nkv, hd, k1, v1, kv.table, page)
+    apart = torch.empty(R, nh * hd, dtype=BF16, device=DEV)
+    _ops.paged_attention(apart, q, k1, v1, kv.table, ctx, nh, nkv, hd, page, scale, window)
+    # plain attention over the cache they left
+    k_h, v_h = k1.cpu().float(), v1.cpu().float()
+    dense = []
+    for r, n in enumerate(kv_lens):
+        pages = [table[r, b].item() for b in range(-(-n // page))]
+        dense.append((torch.cat([k_h[pg].transpose(0, 1) for pg in pages])[:n], torch.cat([v_h[pg].permute(2, 0, 1) for pg in pages])[:n]))
+    qs = [q[r].float().cpu().reshape(1, nh, hd) for r in range(R)]
+    want = dense_attention(qs, dense, [1] * R, kv_lens, scale, window or None).reshape(R, nh * hd)
+    close(apart, want, 2 ** -7, "the separate kernels")
+
+    k2, v2 = kv.k.clone(), kv.v.clone()
+    got = torch.full((R, nh * hd), 7.0, dtype=BF16, device=DEV)
+    assert _ops.decode_attention_from_projection(got, qkv, ctx, rotary, nh, nkv, hd, k2, v2, kv.table, page, scale, window, True)
+    assert torch.equal(k2, k1) and torch.equal(v2, v1), "the cache differs"
+    assert not torch.equal(k2, kv.k), "nothing was written"
+    close(got, want, 2 ** -7, "one kernel")
+    assert torch.equal(got, apart), "a step of single tokens must not depend on which kernels ran it"
+    # without the cache write (a layer that reads another layer's cache): queries only, keys from the cache
+    got2 = torch.full((R, nh * hd), 7.0, dtype=BF16, device=DEV)
+    k3 = k2.clone()
+    assert _ops.decode_attention_from_projection(got2, qkv, ctx, rotary, nh, nkv, hd, k3, v2, kv.table, page, scale, window, False)
+    assert torch.equal(got2, apart) and torch.equal(k3, k2)
+
+
+def test_decode_attention_from_projection_declines_what_it_does_not_serve(_ops):
+    hd, nh, nkv, page = 64, 4, 2, 16
+    seqs = [(torch.randn(20, nkv, hd), torch.randn(20, nkv, hd))] * 2
+    kv = PagedKV(seqs, page, BF16)
+    qkv = torch.randn(2, (nh + 2 * nkv) * hd).to(BF16).to(DEV)
+    out = torch.empty(2, nh * hd, dtype=BF16, device=DEV)
+    inv = torch.ones(16, dtype=F32, device=DEV)
+    # rotation over a part of the head
+    ctx = attention_ctx([1, 1], [20, 20], BF16)
+    assert not _ops.decode_attention_from_projection(out, qkv, ctx, (inv, 32, False), nh, nkv, hd, kv.k, kv.v, kv.table, page, 0.1, 0, True)
+    # a step with a prompt portion
+    ctx = attention_ctx([2, 1], [20, 20], BF16)
+    qkv3 = torch.randn(3, (nh + 2 * nkv) * hd).to(BF16).to(DEV)
+    out3 = torch.empty(3, nh * hd, dtype=BF16, device=DEV)
+    assert not _ops.decode_attention_from_projection(out3, qkv3, ctx, None, nh, nkv, hd, kv.k, kv.v, kv.table, page, 0.1, 0, True)
+
+
 # ------------------------------------------------------------------ attention over pages
 def dense_attention(qs, kvs, q_lens, kv_lens, scale, window):
     """Plain attention per request: the queries are the last q_len positions of kv_len keys."""
