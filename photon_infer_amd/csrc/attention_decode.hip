@@ -36,8 +36,8 @@ struct DecodeSource {
 
 // Values of a token's row of the projection: NO runs of eight consecutive columns (from
 // ocol[i], multiples of 8; rows are 16-byte aligned) and NS single columns, zeros where the
-// lane's flag says so.  Pieces are added in split order, four splits' loads in flight for all
-// columns at once: a wave waits for memory once per four splits, not once per column.
+// lane's flag says so.  Pieces are added in split order, several splits' loads in flight for
+// all columns at once: a wave waits for memory once per group of splits, not once per column.
 template <int NO, int NS>
 __device__ inline void source_gather(const DecodeSource& src, long row, const int (&ocol)[NO], bool octets_wanted,
                                      float (&xo)[NO][8], const int (&scol)[NS > 0 ? NS : 1], bool singles_wanted,
@@ -51,11 +51,12 @@ __device__ inline void source_gather(const DecodeSource& src, long row, const in
   for (int i = 0; i < (NS > 0 ? NS : 1); ++i) xs[i] = 0.f;
   if (src.part) {
     const float* base = src.part + row * src.ncols;
-    for (int s0 = 0; s0 < src.splits; s0 += 4) {
-      quad_t lo[4][NO], hi[4][NO];
-      float one[4][NS > 0 ? NS : 1];
+    constexpr int U = NO <= 2 ? 8 : 4;     // splits in flight: as many as the registers hold
+    for (int s0 = 0; s0 < src.splits; s0 += U) {
+      quad_t lo[U][NO], hi[U][NO];
+      float one[U][NS > 0 ? NS : 1];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < U; ++u) {
         const bool in = s0 + u < src.splits;
         const float* p = base + (long)(in ? s0 + u : 0) * src.part_stride;
 #pragma unroll
@@ -67,7 +68,7 @@ __device__ inline void source_gather(const DecodeSource& src, long row, const in
         for (int i = 0; i < NS; ++i) one[u][i] = (in && singles_wanted) ? p[scol[i]] : 0.f;
       }
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
+      for (int u = 0; u < U; ++u) {
 #pragma unroll
         for (int o = 0; o < NO; ++o)
 #pragma unroll
@@ -242,21 +243,11 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2
   }
 }
 
-// Merge the key ranges of every (request, head): one wave per pair, lane d owns feature d
-// (and d + 64).  Ranges are added in range order; an empty range (m = -inf) counts nothing.
+// Merge the key ranges of one (request, head) by one wave: lane d owns feature d (and d + 64).
+// Ranges are added in range order; an empty range (m = -inf) counts nothing.
 template <int HD>
-__global__ __launch_bounds__(64) void attention_combine_kernel(bf16_t* __restrict__ out, long out_stride,
-                                                               const int* __restrict__ q_start,
-                                                               const int* __restrict__ req_ids,
-                                                               const int* __restrict__ rows,
-                                                               const float* __restrict__ part, int nh, int splits) {
-  const int lane = threadIdx.x;
-  const int head = blockIdx.x;
-  // where the result goes: the token row of request r (decode), or a listed row (cut tiles)
-  const int r = req_ids ? req_ids[blockIdx.y] : (int)blockIdx.y;
-  const long out_row = rows ? rows[blockIdx.y] : q_start[r];
+__device__ inline void combine_ranges(bf16_t* __restrict__ o, const float* base, int splits, int lane) {
   const int rec = HD + 4;
-  const float* base = part + ((long)blockIdx.y * nh + head) * splits * rec;
   // lane s holds range s (splits <= 64): maxima, weights and the total in parallel
   const float ms = lane < splits ? base[lane * rec + HD] : -INFINITY;
   const float ls = lane < splits ? base[lane * rec + HD + 1] : 0.f;
@@ -268,26 +259,40 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(bf16_t* __restric
   for (int i = 0; i < HD / 64; ++i) acc[i] = 0.f;
   // ranges in order; eight loads in flight at a time
   for (int s0 = 0; s0 < splits; s0 += 8) {
-    float o[8][HD / 64], ws[8];
+    float ov[8][HD / 64], ws[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int s = s0 + u;
       ws[u] = __shfl(w, s < splits ? s : 0, 64);
       if (s >= splits) ws[u] = 0.f;
 #pragma unroll
-      for (int i = 0; i < HD / 64; ++i) o[u][i] = (s < splits) ? base[s * rec + lane + i * 64] : 0.f;
+      for (int i = 0; i < HD / 64; ++i) ov[u][i] = (s < splits) ? base[s * rec + lane + i * 64] : 0.f;
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       l_tot += ws[u] * __shfl(ls, (s0 + u < splits) ? s0 + u : 0, 64);
 #pragma unroll
-      for (int i = 0; i < HD / 64; ++i) acc[i] += ws[u] * o[u][i];
+      for (int i = 0; i < HD / 64; ++i) acc[i] += ws[u] * ov[u][i];
     }
   }
   const float inv = 1.0f / l_tot;
-  bf16_t* o = out + out_row * out_stride + (long)head * HD;
 #pragma unroll
   for (int i = 0; i < HD / 64; ++i) o[lane + i * 64] = from_float<bf16_t>(acc[i] * inv);
+}
+
+// One wave per (request, head).
+template <int HD>
+__global__ __launch_bounds__(64) void attention_combine_kernel(bf16_t* __restrict__ out, long out_stride,
+                                                               const int* __restrict__ q_start,
+                                                               const int* __restrict__ req_ids,
+                                                               const int* __restrict__ rows,
+                                                               const float* __restrict__ part, int nh, int splits) {
+  const int head = blockIdx.x;
+  // where the result goes: the token row of request r (decode), or a listed row (cut tiles)
+  const int r = req_ids ? req_ids[blockIdx.y] : (int)blockIdx.y;
+  const long out_row = rows ? rows[blockIdx.y] : q_start[r];
+  combine_ranges<HD>(out + out_row * out_stride + (long)head * HD, part + ((long)blockIdx.y * nh + head) * splits * (HD + 4),
+                     splits, threadIdx.x);
 }
 
 // part: float32 [R * nh * splits * (hd + 4)], needed when splits > 1.
