@@ -77,6 +77,91 @@ __global__ void rmsnorm_kernel(TO* __restrict__ out, float* __restrict__ x, cons
   for (int i = threadIdx.x; i < D; i += blockDim.x) o[i] = from_float<TO>(to_float(w[i]) * (xr[i] * inv));
 }
 
+// The same for rows of a multiple of 4 floats, 16-byte aligned: a thread keeps its VPT groups of
+// four values in registers between the two passes, and every access is 16 bytes wide (8 for
+// bfloat16 output and weights).
+template <typename T> struct Vec4Of;
+template <> struct Vec4Of<float> {
+  typedef float4 type;
+  __device__ static inline void load(const float* p, float (&v)[4]) { const float4 t = *reinterpret_cast<const float4*>(p); v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+  __device__ static inline void store(float* p, const float (&v)[4]) { *reinterpret_cast<float4*>(p) = make_float4(v[0], v[1], v[2], v[3]); }
+};
+template <> struct Vec4Of<bf16_t> {
+  __device__ static inline void load(const bf16_t* p, float (&v)[4]) {
+    const uint2 t = *reinterpret_cast<const uint2*>(p);
+    v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u);
+    v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+  }
+  __device__ static inline void store(bf16_t* p, const float (&v)[4]) {
+    *reinterpret_cast<uint2*>(p) = make_uint2(f32x2_to_bf16x2_bits(v[0], v[1]), f32x2_to_bf16x2_bits(v[2], v[3]));
+  }
+};
+
+template <typename TO, typename TW, int VPT>
+__global__ void rmsnorm_wide_kernel(TO* __restrict__ out, float* __restrict__ x, const int* __restrict__ rows,
+                                    const TW* __restrict__ w, float eps, int D, const float* __restrict__ part, int splits,
+                                    long part_stride) {
+  __shared__ float scratch[16];
+  const long m = blockIdx.x;
+  const long r = rows ? rows[m] : m;
+  float* xr = x + r * D;
+  const int groups = D / 4;
+  float v[VPT][4], ww[VPT][4];      // the weights come along with the row: one wait for memory, not two
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int gi = threadIdx.x + k * blockDim.x;
+    if (gi < groups) {
+      Vec4Of<float>::load(xr + gi * 4, v[k]);
+      Vec4Of<TW>::load(w + gi * 4, ww[k]);
+    } else {
+      v[k][0] = v[k][1] = v[k][2] = v[k][3] = 0.f;
+      ww[k][0] = ww[k][1] = ww[k][2] = ww[k][3] = 0.f;
+    }
+  }
+  if (part) {
+    const float* pr = part + r * D;
+    for (int s0 = 0; s0 < splits; s0 += 4) {     // four pieces' loads go out together, the adds keep the split order
+      float t[4][VPT][4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+          const int gi = threadIdx.x + k * blockDim.x;
+          if (s0 + u < splits && gi < groups) Vec4Of<float>::load(pr + (s0 + u) * part_stride + gi * 4, t[u][k]);
+          else t[u][k][0] = t[u][k][1] = t[u][k][2] = t[u][k][3] = 0.f;
+        }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+#pragma unroll
+        for (int k = 0; k < VPT; ++k)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[k][e] += t[u][k][e];
+    }
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      const int gi = threadIdx.x + k * blockDim.x;
+      if (gi < groups) Vec4Of<float>::store(xr + gi * 4, v[k]);
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) ss += v[k][e] * v[k][e];
+  ss = block_sum(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)D + eps);
+  TO* o = out + m * D;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int gi = threadIdx.x + k * blockDim.x;
+    if (gi >= groups) continue;
+    float y[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) y[e] = ww[k][e] * (v[k][e] * inv);
+    Vec4Of<TO>::store(o + gi * 4, y);
+  }
+}
+
 // part == nullptr: plain norm.  Otherwise part is float32 [splits, x_rows, D].
 extern "C" int pi_rmsnorm(void* out, int out_dtype, float* x, const int* rows, const void* w, int w_dtype, float eps, int M,
                           int D, const float* part, int splits, long x_rows, hipStream_t stream) {
@@ -84,16 +169,36 @@ extern "C" int pi_rmsnorm(void* out, int out_dtype, float* x, const int* rows, c
   PI_REQUIRE(part == nullptr || (splits >= 1 && x_rows > 0), "rmsnorm: bad split description (%d splits, %ld rows)", splits, x_rows);
   if (M == 0) return 0;
   // few rows: many threads per row, so that a row's loads are all in flight at once
-  const int threads = (D >= 2048 && M <= 256) ? 1024 : (D >= 1024 ? 256 : (D >= 256 ? 128 : 64));
+  int threads = (D >= 2048 && M <= 256) ? 1024 : (D >= 1024 ? 256 : (D >= 256 ? 128 : 64));
   const long stride = x_rows * (long)D;
+  // rows of whole 16-byte groups, at most 8 groups per thread: the kernel with wide accesses
+  // (no more threads than groups)
+  bool wide = D % 4 == 0 && ((uintptr_t)x % 16 == 0) && ((uintptr_t)out % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
+              (part == nullptr || (uintptr_t)part % 16 == 0);
+  int per_thread = 0;
+  if (wide) {
+    const int groups = D / 4, most = threads;
+    threads = groups >= most ? most : ((groups + 63) / 64) * 64;
+    per_thread = (groups + threads - 1) / threads;
+    if (per_thread > 8) { wide = false; threads = most; }
+  }
+#define WIDE(TO, TW, V) \
+  hipLaunchKernelGGL((rmsnorm_wide_kernel<TO, TW, V>), dim3(M), dim3(threads), 0, stream, (TO*)out, x, rows, (const TW*)w, eps, D, part, splits, stride)
 #define LAUNCH(TO, TW) \
-  hipLaunchKernelGGL((rmsnorm_kernel<TO, TW>), dim3(M), dim3(threads), 0, stream, (TO*)out, x, rows, (const TW*)w, eps, D, part, splits, stride)
+  do { \
+    if (wide && per_thread <= 1) WIDE(TO, TW, 1); \
+    else if (wide && per_thread <= 2) WIDE(TO, TW, 2); \
+    else if (wide && per_thread <= 4) WIDE(TO, TW, 4); \
+    else if (wide) WIDE(TO, TW, 8); \
+    else hipLaunchKernelGGL((rmsnorm_kernel<TO, TW>), dim3(M), dim3(threads), 0, stream, (TO*)out, x, rows, (const TW*)w, eps, D, part, splits, stride); \
+  } while (0)
   if (out_dtype == PI_F32 && w_dtype == PI_F32) LAUNCH(float, float);
   else if (out_dtype == PI_F32 && w_dtype == PI_BF16) LAUNCH(float, bf16_t);
   else if (out_dtype == PI_BF16 && w_dtype == PI_F32) LAUNCH(bf16_t, float);
   else if (out_dtype == PI_BF16 && w_dtype == PI_BF16) LAUNCH(bf16_t, bf16_t);
   else return pi_fail("rmsnorm: unsupported dtypes out=%d weight=%d", out_dtype, w_dtype);
 #undef LAUNCH
+#undef WIDE
   return pi_check_launch("rmsnorm");
 }
 
