@@ -48,7 +48,17 @@ TINY_D = dict(
 )
 TINY_D_INIT = dict(std=0.08, norm_init="uniform", block_size=16)
 
-ALL = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT), "D": (TINY_D, TINY_D_INIT)}
+# the other head size of the matrix-core kernels (128), four heads on one kv head, pages of 32,
+# an untied head, no scaling of the rotation
+TINY_E = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=160, intermediate_size=344, num_hidden_layers=2,
+    num_attention_heads=4, num_key_value_heads=1, head_dim=128, vocab_size=776, max_position_embeddings=512,
+    rms_norm_eps=1e-6, rope_theta=10000.0, tie_word_embeddings=False,
+)
+TINY_E_INIT = dict(std=0.06, norm_init="uniform", block_size=32)
+
+ALL = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT), "D": (TINY_D, TINY_D_INIT),
+       "E": (TINY_E, TINY_E_INIT)}
 
 
 def make_model_dir(tmp_path, name: str, seed: int = 0, storage: str = "bfloat16") -> str:
