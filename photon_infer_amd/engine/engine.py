@@ -51,6 +51,8 @@ class ContinuousBatchEngine:
         self.steps = 0
         # a decode step that was launched and whose tokens have not been read yet
         self._in_flight: Optional[_InFlight] = None
+        # pinned buffers the sampled tokens are copied to, by (batch size, turn)
+        self._buffers: Dict[tuple, "torch.Tensor"] = {}
 
     @property
     def config(self):
@@ -115,10 +117,8 @@ class ContinuousBatchEngine:
         import torch
         # two pinned buffers per size, used in turn: one is still being read when the next copy starts
         key = (n, self.steps % 2)
-        buf = self._buffers.get(key) if hasattr(self, "_buffers") else None
+        buf = self._buffers.get(key)
         if buf is None:
-            if not hasattr(self, "_buffers"):
-                self._buffers = {}
             buf = self._buffers[key] = torch.empty(n, dtype=torch.int32, pin_memory=True)
         return buf
 
