@@ -34,10 +34,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
   const int lane = threadIdx.x % 64;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
   const int lr = lane % 16, lg = lane / 16;
-  const int g = blockIdx.y, G = nh / nkv, B = gridDim.x;
-  // blocks of the second half of the kv heads take the deal in reverse: two blocks that end
-  // up on one compute unit then tend to hold a long and a short tile
-  const int seat = (2 * blockIdx.y >= gridDim.y) ? B - 1 - (int)blockIdx.x : (int)blockIdx.x;
+  // kv head in x: with 8 kv heads (or a multiple) a die, which takes every eighth block, walks
+  // the keys of one kv head only and its L2 serves all tiles of that head
+  const int g = blockIdx.x, G = nh / nkv, B = gridDim.y;
+  // The host deals long tiles to low seats.  A die's 32 compute units take its blocks in turn,
+  // so blocks y and y + 32 meet on one unit: every other run of 32 takes its seats in reverse,
+  // and a long tile sits beside a short one.
+  const int run = blockIdx.y / 32, run_len = min(32, B - run * 32);
+  const int seat = run * 32 + ((run & 1) ? run_len - 1 - (int)(blockIdx.y % 32) : (int)(blockIdx.y % 32));
   const int num_pages = (int)(num_pages_l < 0x7fffffffL ? num_pages_l : 0x7fffffffL);
   const float scale_log2 = scale * PI_LOG2E;
   KVLaneOffsets<HD> off;
@@ -212,7 +216,7 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
     if (e != hipSuccess) return pi_fail("attention_prefill: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     configured[hd == 128] = true;
   }
-  const dim3 grid(seats, nkv), block(256);
+  const dim3 grid(nkv, seats), block(256);
 #define GO(H, C) hipLaunchKernelGGL((attention_tiles_kernel<H, C>), grid, block, lds, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, \
                                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, \
                                     kv_len, tile_req, tile_q0, tile_cut, tile_z0, (float*)part, order, rounds, nh, nkv, page_size, scale, \
