@@ -344,8 +344,8 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
   }
 }
 
-// The same for the common case, many tokens at a time (prompts): bfloat16 tensors (no pieces),
-// rotation over the whole head with halves paired, head size a multiple of 16.  Every memory
+// The same for the common case, many tokens at a time (prompts): bfloat16 tensors or float32
+// pieces, rotation over the whole head with halves paired, head size a multiple of 16.  Every memory
 // access is wide: a thread turns 8 features and their 8 partners of one (token, head) (16-byte
 // loads and stores, in place for queries, into the page for keys); for values a thread takes
 // one feature of four consecutive tokens and, when the four are neighbours in one page,
@@ -354,7 +354,8 @@ __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
     bf16_t* __restrict__ q, long q_stride, const bf16_t* __restrict__ k, long k_stride, const bf16_t* __restrict__ v,
     long v_stride, const int* __restrict__ positions, const int* __restrict__ req_of_token, const float* __restrict__ table,
     int rotate, int T, int nh, int nkv_write, int nkv, int hd, bf16_t* __restrict__ k_cache, bf16_t* __restrict__ v_cache,
-    const int* __restrict__ block_table, int table_width, int page_size, long num_pages, long rot_items) {
+    const int* __restrict__ block_table, int table_width, int page_size, long num_pages, long rot_items,
+    const float* __restrict__ part, int splits, long part_stride, int ncols, int q_col, int k_col, int v_col) {
   const long idx = (long)blockIdx.x * 256 + threadIdx.x;
   const int units = hd / 16, heads = nh + nkv_write;
   if (idx < rot_items) {
@@ -363,9 +364,11 @@ __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
     const int d = unit * 8;                      // features d .. d + 7 and their partners at + hd / 2
     const bf16_t* src;
     bf16_t* dst;
+    int col;                                     // the head's first column among the pieces
     if (head < nh) {
       dst = q + t * q_stride + (long)head * hd;
       src = dst;
+      col = q_col + head * hd;
     } else {
       const int g = head - nh, pos = positions[t], blk = pos / page_size;
       if (blk >= table_width) return;
@@ -373,38 +376,58 @@ __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
       if (page < 0 || page >= num_pages) return;   // the host checks tables; never write outside the pool
       src = k + t * k_stride + (long)g * hd;
       dst = k_cache + ((page * nkv + g) * page_size + (pos % page_size)) * hd;
+      col = k_col + g * hd;
     }
-    if (!rotate && dst == src) return;
-    const uint4 lo = *reinterpret_cast<const uint4*>(src + d), hi = *reinterpret_cast<const uint4*>(src + d + hd / 2);
-    uint4 out_lo = lo, out_hi = hi;
+    if (!part && !rotate && dst == src) return;
+    typedef float quad_t __attribute__((ext_vector_type(4)));
+    float a[8], b[8];                            // the features and their partners, float32
+    if (part) {
+#pragma unroll
+      for (int e = 0; e < 8; ++e) a[e] = b[e] = 0.f;
+      const float* p = part + t * ncols + col + d;
+      for (int s0 = 0; s0 < splits; s0 += 4) {   // four pieces' loads go out together, the adds keep the split order
+        quad_t la[4][2], lb[4][2];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const bool in = s0 + u < splits;
+          const float* ps = p + (long)(in ? s0 + u : 0) * part_stride;
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            la[u][h] = in ? *reinterpret_cast<const quad_t*>(ps + 4 * h) : quad_t{0.f, 0.f, 0.f, 0.f};
+            lb[u][h] = in ? *reinterpret_cast<const quad_t*>(ps + hd / 2 + 4 * h) : quad_t{0.f, 0.f, 0.f, 0.f};
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+          for (int e = 0; e < 8; ++e) { a[e] += la[u][e / 4][e % 4]; b[e] += lb[u][e / 4][e % 4]; }
+      }
+    } else {
+      const uint4 lo = *reinterpret_cast<const uint4*>(src + d), hi = *reinterpret_cast<const uint4*>(src + d + hd / 2);
+      const uint32_t lw[4] = {lo.x, lo.y, lo.z, lo.w}, hw[4] = {hi.x, hi.y, hi.z, hi.w};
+#pragma unroll
+      for (int w = 0; w < 4; ++w) {              // two features per 32-bit word
+        a[2 * w] = __uint_as_float(lw[w] << 16); a[2 * w + 1] = __uint_as_float(lw[w] & 0xffff0000u);
+        b[2 * w] = __uint_as_float(hw[w] << 16); b[2 * w + 1] = __uint_as_float(hw[w] & 0xffff0000u);
+      }
+    }
     if (rotate) {
       const float* c = table + t * hd + d;
       const float* sn = c + hd / 2;
-      typedef float quad_t __attribute__((ext_vector_type(4)));
       const quad_t c0 = *reinterpret_cast<const quad_t*>(c), c1 = *reinterpret_cast<const quad_t*>(c + 4);
       const quad_t s0 = *reinterpret_cast<const quad_t*>(sn), s1 = *reinterpret_cast<const quad_t*>(sn + 4);
-      const uint32_t* lw = reinterpret_cast<const uint32_t*>(&lo);
-      const uint32_t* hw = reinterpret_cast<const uint32_t*>(&hi);
-      uint32_t ol[4], oh[4];
 #pragma unroll
-      for (int w = 0; w < 4; ++w) {              // two features per 32-bit word
-        float a[2] = {__uint_as_float(lw[w] << 16), __uint_as_float(lw[w] & 0xffff0000u)};
-        float b[2] = {__uint_as_float(hw[w] << 16), __uint_as_float(hw[w] & 0xffff0000u)};
-        float rl[2], rh[2];
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          const int i = 2 * w + e;
-          const float cc = i < 4 ? c0[i] : c1[i - 4], ss = i < 4 ? s0[i] : s1[i - 4];
-          rope_pair(a[e], b[e], cc, ss, rl[e], rh[e]);
-        }
-        ol[w] = f32x2_to_bf16x2_bits(rl[0], rl[1]);
-        oh[w] = f32x2_to_bf16x2_bits(rh[0], rh[1]);
+      for (int e = 0; e < 8; ++e) {
+        float lo_e, hi_e;
+        rope_pair(a[e], b[e], e < 4 ? c0[e] : c1[e - 4], e < 4 ? s0[e] : s1[e - 4], lo_e, hi_e);
+        a[e] = lo_e;
+        b[e] = hi_e;
       }
-      out_lo = make_uint4(ol[0], ol[1], ol[2], ol[3]);
-      out_hi = make_uint4(oh[0], oh[1], oh[2], oh[3]);
     }
-    *reinterpret_cast<uint4*>(dst + d) = out_lo;
-    *reinterpret_cast<uint4*>(dst + d + hd / 2) = out_hi;
+    *reinterpret_cast<uint4*>(dst + d) = make_uint4(f32x2_to_bf16x2_bits(a[0], a[1]), f32x2_to_bf16x2_bits(a[2], a[3]),
+                                                    f32x2_to_bf16x2_bits(a[4], a[5]), f32x2_to_bf16x2_bits(a[6], a[7]));
+    *reinterpret_cast<uint4*>(dst + d + hd / 2) = make_uint4(f32x2_to_bf16x2_bits(b[0], b[1]), f32x2_to_bf16x2_bits(b[2], b[3]),
+                                                             f32x2_to_bf16x2_bits(b[4], b[5]), f32x2_to_bf16x2_bits(b[6], b[7]));
     return;
   }
   // values: (four tokens, kv head, feature)
@@ -418,7 +441,12 @@ __global__ __launch_bounds__(256) void rope_kv_write_wide_kernel(
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     const long t = t0 + (i < n ? i : 0);
-    val[i] = *reinterpret_cast<const uint16_t*>(v + t * v_stride + (long)g * hd + d);
+    if (part) {
+      const bf16_t r = from_float<bf16_t>(split_sum(part, splits, part_stride, t * ncols + v_col + g * hd + d));
+      val[i] = *reinterpret_cast<const uint16_t*>(&r);
+    } else {
+      val[i] = *reinterpret_cast<const uint16_t*>(v + t * v_stride + (long)g * hd + d);
+    }
     pos[i] = positions[t];
     req[i] = req_of_token[t];
   }
@@ -462,10 +490,11 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
   if (T == 0 || heads == 0) return 0;
   // many bfloat16 tokens with the usual rotation: the kernel with wide accesses
   const bool usual = rotary_dim == 0 || (rotary_dim == hd && !interleaved);
+  const bool source_ok = part ? (ncols % 4 == 0 && ((uintptr_t)part % 16 == 0) && q_col % 4 == 0 && k_col % 4 == 0)
+                              : (!write_kv || (k_stride % 8 == 0 && ((uintptr_t)k % 16 == 0)));
   const bool aligned = hd % 16 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && (!table || (uintptr_t)table % 16 == 0) &&
-                       (!write_kv || (k_stride % 8 == 0 && ((uintptr_t)k % 16 == 0) && ((uintptr_t)k_cache % 16 == 0) &&
-                                      ((uintptr_t)v_cache % 8 == 0) && page_size % 4 == 0));
-  if (dtype == PI_BF16 && !part && usual && aligned && T >= 16) {
+                       source_ok && (!write_kv || (((uintptr_t)k_cache % 16 == 0) && ((uintptr_t)v_cache % 8 == 0) && page_size % 4 == 0));
+  if (dtype == PI_BF16 && usual && aligned && T >= 16) {
     const int nkv_w = write_kv ? nkv : 0;
     const long rot_items = (long)T * (nh + nkv_w) * (hd / 16);
     const long v_items = write_kv ? (long)((T + 3) / 4) * nkv * hd : 0;
@@ -474,7 +503,7 @@ extern "C" int pi_rope_kv_write(void* q, long q_stride, const void* k, long k_st
     hipLaunchKernelGGL(rope_kv_write_wide_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, (bf16_t*)q, q_stride,
                        (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, positions, req_of_token, table,
                        rotary_dim > 0 ? 1 : 0, T, nh, nkv_w, nkv, hd, (bf16_t*)k_cache, (bf16_t*)v_cache, block_table,
-                       table_width, page_size, num_pages, rot_items);
+                       table_width, page_size, num_pages, rot_items, part, splits, (long)T * ncols, ncols, q_col, k_col, v_col);
     return pi_check_launch("rope_kv_write_wide");
   }
   PI_REQUIRE(heads <= 65535, "rope_kv_write: too many heads (%d)", heads);

@@ -266,18 +266,30 @@ def test_rope_kv_write(_ops, dtype, hd, rot, inter):
 
 
 @pytest.mark.parametrize("hd,page,rotate", [(64, 16, True), (128, 4, True), (64, 8, False), (16, 4, True)])
-def test_rope_kv_write_many_tokens(_ops, hd, page, rotate):
+@pytest.mark.parametrize("pieces", [0, 3, 6])
+def test_rope_kv_write_many_tokens(_ops, hd, page, rotate, pieces):
     """Prompts take the kernel with wide accesses: portions that start at any row of the batch
-    and at any position, single tokens among them, pages of several sizes."""
+    and at any position, single tokens among them, pages of several sizes; q, k and v as a
+    bfloat16 tensor or as float32 pieces of a product split over k (summed in float32, rounded
+    once after the rotation)."""
     nh, nkv, dtype = 4, 2, BF16
     q_lens, kv_lens = [40, 1, 23, 7, 16], [40, 30, 55, 19, 48]    # whole, decode, later portions (rows 41.., 64.., 71..)
     R, T = len(q_lens), sum(q_lens)
     ctx = attention_ctx(q_lens, kv_lens, dtype)
     freqs = P.rope_frequencies(hd, 10000.0, None)
     inv = torch.tensor(freqs, dtype=torch.float64).to(F32).to(DEV)
-    qkv = torch.randn(T, (nh + 2 * nkv) * hd, generator=gen(hd + page)).to(dtype)
-    dev = qkv.to(DEV)
-    q, k, v = dev[:, :nh * hd], dev[:, nh * hd:(nh + nkv) * hd], dev[:, (nh + nkv) * hd:]
+    if pieces:
+        from photon_infer_amd.ops import fast
+        part = torch.randn(pieces, T, (nh + 2 * nkv) * hd, generator=gen(hd + page)) * 0.5
+        qkv = part[0].clone()
+        for s_ in range(1, pieces):       # the kernel's order of adding
+            qkv += part[s_]
+        source = fast.Partials(part.to(DEV), pieces, T, (nh + 2 * nkv) * hd)
+        q = torch.empty(T, nh * hd, dtype=dtype, device=DEV)
+    else:
+        qkv = torch.randn(T, (nh + 2 * nkv) * hd, generator=gen(hd + page)).to(dtype)
+        dev = qkv.to(DEV)
+        q, k, v = dev[:, :nh * hd], dev[:, nh * hd:(nh + nkv) * hd], dev[:, (nh + nkv) * hd:]
     blocks = [-(-kv // page) for kv in kv_lens]
     pages = sum(blocks) + 3
     order = torch.randperm(pages, generator=gen(11)).tolist()
@@ -288,8 +300,12 @@ def test_rope_kv_write_many_tokens(_ops, hd, page, rotate):
             table[r, b] = next(it)
     kc = torch.zeros(pages, nkv, page, hd, dtype=dtype, device=DEV)
     vc = torch.zeros(pages, nkv, hd, page, dtype=dtype, device=DEV)
-    _ops.rope_kv_write(q, k, v, ctx.positions, ctx.req_of_token, (inv, hd, False) if rotate else None, nh, nkv, hd, kc, vc,
-                       table.to(DEV), page)
+    if pieces:
+        _ops.rope_kv_write(q, None, None, ctx.positions, ctx.req_of_token, (inv, hd, False) if rotate else None, nh, nkv, hd,
+                           kc, vc, table.to(DEV), page, pieces=source, write_kv=True)
+    else:
+        _ops.rope_kv_write(q, k, v, ctx.positions, ctx.req_of_token, (inv, hd, False) if rotate else None, nh, nkv, hd, kc, vc,
+                           table.to(DEV), page)
     pos = ctx.positions.cpu().tolist()
     req = ctx.req_of_token.cpu().tolist()
     turn = (lambda x: P.rope(x, pos, freqs, False)) if rotate else (lambda x: x)
@@ -303,7 +319,7 @@ def test_rope_kv_write_many_tokens(_ops, hd, page, rotate):
         pg, sl = table[req[t], pos[t] // page].item(), pos[t] % page
         written[pg, sl] = True
         close(kc_h[pg, :, sl], k_want[t], 2 ** -8, f"k of token {t}")
-        assert torch.equal(vc_h[pg, :, :, sl], v_want[t]), f"v of token {t}"
+        assert torch.equal(vc_h[pg, :, :, sl], v_want[t].to(dtype).float()), f"v of token {t}"
     assert kc_h[~written.unsqueeze(1).expand(-1, nkv, -1)].abs().max() == 0
     assert vc_h.permute(0, 1, 3, 2)[~written.unsqueeze(1).expand(-1, nkv, -1)].abs().max() == 0
 
