@@ -29,9 +29,6 @@ struct DecodeSource {
   int write_kv;
   bf16_t* k_cache;
   bf16_t* v_cache;
-  __device__ inline float at(long row, int col) const {
-    return part ? split_sum(part, splits, part_stride, row * ncols + col) : to_float(qkv[row * qkv_stride + col]);
-  }
 };
 
 // Values of a token's row of the projection: NO runs of eight consecutive columns (from
