@@ -52,17 +52,26 @@ __device__ inline void source_gather(const DecodeSource& src, long row, const in
     for (int s0 = 0; s0 < src.splits; s0 += U) {
       quad_t lo[U][NO], hi[U][NO];
       float one[U][NS > 0 ? NS : 1];
+      // every load is made (a split beyond the last reads the first again, a lane that wants
+      // nothing reads column 0) and what is not wanted is zeroed afterwards: no branch around
+      // each load, a fraction of the code
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const bool in = s0 + u < src.splits;
         const float* p = base + (long)(in ? s0 + u : 0) * src.part_stride;
+        const quad_t zero = quad_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
         for (int o = 0; o < NO; ++o) {
-          lo[u][o] = (in && octets_wanted) ? *reinterpret_cast<const quad_t*>(p + ocol[o]) : quad_t{0.f, 0.f, 0.f, 0.f};
-          hi[u][o] = (in && octets_wanted) ? *reinterpret_cast<const quad_t*>(p + ocol[o] + 4) : quad_t{0.f, 0.f, 0.f, 0.f};
+          const int c = octets_wanted ? ocol[o] : 0;
+          const quad_t l = *reinterpret_cast<const quad_t*>(p + c), h = *reinterpret_cast<const quad_t*>(p + c + 4);
+          lo[u][o] = (in && octets_wanted) ? l : zero;
+          hi[u][o] = (in && octets_wanted) ? h : zero;
         }
 #pragma unroll
-        for (int i = 0; i < NS; ++i) one[u][i] = (in && singles_wanted) ? p[scol[i]] : 0.f;
+        for (int i = 0; i < NS; ++i) {
+          const float v = p[singles_wanted ? scol[i] : 0];
+          one[u][i] = (in && singles_wanted) ? v : 0.f;
+        }
       }
 #pragma unroll
       for (int u = 0; u < U; ++u) {
