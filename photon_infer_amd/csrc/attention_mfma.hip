@@ -205,7 +205,7 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
   PI_REQUIRE(table_width >= 1, "attention_prefill: empty block table");
   const int TQ = pi_attention_tile_rows(nh, nkv, hd);
   PI_REQUIRE(TQ >= 1, "attention_prefill: %d heads per kv head do not fit a block", nh / nkv);
-  PI_REQUIRE(nkv <= 65535, "attention_prefill: too many kv heads (%d)", nkv);
+  PI_REQUIRE(seats <= 65535, "attention_prefill: too many blocks per kv head (%d)", seats);
   PI_REQUIRE(out_stride % 4 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "attention_prefill: q / out rows must be 16- / 8-byte aligned");
   const size_t lds = tiles_lds_bytes(hd);
   static bool configured[2] = {false, false};
