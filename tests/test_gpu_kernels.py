@@ -559,3 +559,82 @@ def test_temperature_sampling_frequencies_and_limits(_ops):
     # a tiny temperature is the argmax; u near 1 still lands on a token with p > 0
     _ops.sample(out[:2], l[:2].to(DEV), torch.full((2,), 1e-4, device=DEV), torch.tensor([0.3, 0.9999999], device=DEV))
     assert out[:2].cpu().tolist() == [2, 2]
+
+
+# ------------------------------------------------------------------ sampling from large vocabularies (two kernels)
+def _sample_chunk(V):
+    """Length of the chunks a row of V logits is cut into (0: rows this short take one kernel)."""
+    from photon_infer_amd.ops import _lib
+    chunks = _lib.load("core").pi_sample_chunks(V)
+    return -(-V // chunks) if chunks else 0
+
+
+@pytest.mark.parametrize("V", [16385, 50021, 128256])
+def test_temperature_sampling_of_large_vocabularies_matches_the_inverse_cdf(_ops, V):
+    assert _sample_chunk(V) > 0 and _sample_chunk(16384) == 0
+    g = gen(V)
+    M = 24
+    l = torch.randn(M, V, generator=g) * 3
+    temps = torch.full((M,), 0.7)
+    temps[::5] = 0.0                                            # greedy rows beside sampled rows
+    temps[1::5] = 1.9
+    u = torch.rand(M, generator=g)
+    u[2], u[3], u[7] = 0.0, 0.99999994, 1e-7
+    out = torch.empty(M, dtype=torch.int32, device=DEV)
+    _ops.sample(out, l.to(DEV), temps.to(DEV), u.to(DEV))
+    got = out.cpu().tolist()
+    for r in range(M):
+        if temps[r] == 0:
+            assert got[r] == int(l[r].argmax())
+            continue
+        c = torch.cumsum(torch.softmax(l[r].double() / temps[r].item(), 0), 0)
+        lo = c[got[r] - 1].item() if got[r] > 0 else 0.0
+        assert lo - 2e-5 <= u[r].item() <= c[got[r]].item() + 2e-5, (r, got[r], lo, u[r].item(), c[got[r]].item())
+
+
+@pytest.mark.parametrize("V", [16385, 50021, 128256])
+def test_temperature_sampling_at_the_edges_of_chunks(_ops, V):
+    """Rows whose probability sits on a few tokens at chunk edges, so that the draw names its token
+    without doubt: the last token of a chunk and the first of the next, chunks without any weight
+    before, between and after them, the first and the last token of the row."""
+    chunk = _sample_chunk(V)
+    chunks = -(-V // chunk)
+    NEG = float("-inf")
+    rows, draws, want = [], [], []
+
+    def case(weights: dict, u: float, token: int, floor=NEG):
+        row = torch.full((V,), floor)
+        for i, w in weights.items():
+            row[i] = math.log(w)
+        rows.append(row)
+        draws.append(u)
+        want.append(token)
+
+    k = chunks // 2
+    a, b = k * chunk - 1, k * chunk                      # last token of chunk k-1, first of chunk k
+    for u, tok in ((0.25, a), (0.4999, a), (0.5001, b), (0.75, b), (1e-9, a), (0.99999994, b)):
+        case({a: 0.5, b: 0.5}, u, tok)                   # every other chunk holds -inf only
+    # the same with a little weight everywhere (1e-12 in all of the rest together)
+    for u, tok in ((0.25, a), (0.4999, a), (0.5001, b), (0.75, b)):
+        case({a: 0.5, b: 0.5}, u, tok, floor=math.log(1e-12 / V))
+    # first and last token of the row; the last chunk is the short one
+    case({0: 0.3, V - 1: 0.7}, 0.29, 0)
+    case({0: 0.3, V - 1: 0.7}, 0.31, V - 1)
+    case({0: 0.3, V - 1: 0.7}, 0.99999994, V - 1)
+    # three tokens in three different chunks with empty chunks between them
+    x, y, z = 5, (chunks // 3) * chunk + 17, (chunks - 1) * chunk + 1
+    for u, tok in ((0.1, x), (0.21, y), (0.69, y), (0.71, z), (0.95, z)):
+        case({x: 0.2, y: 0.5, z: 0.3}, u, tok)
+    # all the weight in one chunk, spread over the chunk's last 100 tokens
+    lo_tok = 2 * chunk - 100
+    for u in (0.005, 0.505, 0.995):
+        case({lo_tok + i: 0.01 for i in range(100)}, u, lo_tok + int(u * 100))
+    l = torch.stack(rows)
+    for tau in (1.0, 0.5):
+        # at temperature tau the weights are p^(1/tau): feed tau * log p to keep the intended weights
+        out = torch.empty(len(rows), dtype=torch.int32, device=DEV)
+        _ops.sample(out, (l * tau).to(DEV), torch.full((len(rows),), tau, device=DEV), torch.tensor(draws, device=DEV))
+        assert out.cpu().tolist() == want, tau
+    # the plain implementation agrees on the crafted rows (a few of them: it walks the row in Python)
+    for r in (1, 2, 11, 14):
+        assert P.sample_temperature(l[r].double(), 1.0, draws[r]) == want[r]

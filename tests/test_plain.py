@@ -138,6 +138,57 @@ def test_llama3_scaling_hits_all_three_regimes():
     assert all(abs(a - b / 4) < 1e-18 for a, b in zip(lin, base))
 
 
+def _both_frequency_tables(rotary_dim, theta, sc):
+    """The plain implementation's frequencies and the product's, for the same constants."""
+    from photon_infer_amd.config.llama import RopeScaling
+    from photon_infer_amd.parts.rope import rope_frequencies
+
+    plain = P.rope_frequencies(rotary_dim, theta, sc)
+    typed = None if sc is None else RopeScaling(**sc)
+    return (("plain", plain), ("product", rope_frequencies(rotary_dim, theta, typed).tolist()))
+
+
+def test_llama3_blend_falls_from_one_to_one_over_factor():
+    # head size 128 with the constants of the 1B model: six pairs lie in the blended band.  The
+    # ratio scaled / base must fall with the pair index from 1 (short wavelengths are kept) to
+    # 1 / factor.  A blend with its two weights exchanged rises inside the band instead.
+    sc = dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+              original_max_position_embeddings=8192)
+    base = P.rope_frequencies(128, 500000.0, None)
+    lam = [2 * math.pi / b for b in base]
+    mid = [j for j in range(64) if 8192 / 4 <= lam[j] <= 8192 / 1]
+    assert len(mid) >= 5 and mid == list(range(mid[0], mid[-1] + 1))
+    for who, f in _both_frequency_tables(128, 500000.0, sc):
+        ratio = [a / b for a, b in zip(f, base)]
+        assert all(abs(r - 1.0) < 1e-13 for r in ratio[:mid[0]]), who
+        assert all(abs(r - 1 / 32) < 1e-13 for r in ratio[mid[-1] + 1:]), who
+        assert all(ratio[j] > ratio[j + 1] for j in range(mid[0] - 1, mid[-1] + 1)), who
+        assert all(1 / 32 < ratio[j] < 1.0 for j in mid), who
+        # the band's formula: linear in L / wavelength between the two ends
+        for j in mid:
+            s = (8192 / lam[j] - 1.0) / (4.0 - 1.0)
+            assert abs(ratio[j] - ((1 - s) / 32 + s)) < 1e-12, (who, j)
+
+
+def test_llama3_blend_is_continuous_at_both_thresholds():
+    # Move the original context length so that one pair's wavelength sits a hair inside the band at
+    # its short end, then at its long end: the ratio there is (almost) 1 and (almost) 1 / factor.
+    # Exchanged weights give 1 / factor and 1; a band test with "<" for "<=" is caught as well.
+    base = P.rope_frequencies(64, 500000.0, None)
+    j = 20
+    lam = 2 * math.pi / base[j]
+    for L, want in ((lam * 4.0 * (1 + 1e-9), 1.0), (lam * 1.0 * (1 - 1e-9), 1 / 16)):
+        sc = dict(rope_type="llama3", factor=16.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                  original_max_position_embeddings=L)
+        for who, f in _both_frequency_tables(64, 500000.0, sc):
+            assert abs(f[j] / base[j] - want) < 1e-7, (who, L, f[j] / base[j])
+    for L, want in ((lam * 4.0 * (1 - 1e-9), 1.0), (lam * 1.0 * (1 + 1e-9), 1 / 16)):   # a hair outside: the same values
+        sc = dict(rope_type="llama3", factor=16.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                  original_max_position_embeddings=L)
+        for who, f in _both_frequency_tables(64, 500000.0, sc):
+            assert abs(f[j] / base[j] - want) < 1e-7, (who, L, f[j] / base[j])
+
+
 # ------------------------------------------------------------------ attention against a library routine
 def _library_attention(q, k, v, scale, window=None):
     S, nh, hd = q.shape
