@@ -9,6 +9,7 @@
 // the caller, so a request's draws do not depend on what else is in the batch.  If
 // rounding lets the cumulative sum end below u * sum, the last index with p > 0 is taken.
 #include "common.h"
+#include "sampling.h"
 
 #define SAMPLE_THREADS 256
 
@@ -253,4 +254,46 @@ extern "C" int pi_sample(int* out, const float* logits, long row_stride, const f
   if (pi_check_launch("sample_stage1")) return -1;
   hipLaunchKernelGGL(sample_stage2_kernel, dim3(M), dim3(SAMPLE_THREADS), 0, stream, out, ws, logits, row_stride, temperature, uniform, V, chunk, chunks);
   return pi_check_launch("sample_stage2");
+}
+
+// ---- the entry point that allocates nothing: the chunk records live in an array of the library's
+// own.  Each GPU holds its own copy of the array at its own address; in host code the array's
+// name is only a handle for hipGetSymbolAddress, never a pointer a kernel may be given.
+static __device__ __align__(256) float sample_static_records[PI_SAMPLE_STATIC_FLOATS];
+
+#define SAMPLE_MAX_DEVICES 64
+static float* sample_static_ptr[SAMPLE_MAX_DEVICES] = {nullptr};
+
+// The device address of the array on the current GPU (looked up once per GPU, at the first call there).
+static int sample_static_address(float** ptr) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  PI_REQUIRE(e == hipSuccess, "sample_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  PI_REQUIRE(dev >= 0 && dev < SAMPLE_MAX_DEVICES, "sample_static: device %d is beyond the %d this library keeps an address for",
+             dev, SAMPLE_MAX_DEVICES);
+  if (sample_static_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(sample_static_records));
+    PI_REQUIRE(e == hipSuccess && p != nullptr, "sample_static: hipGetSymbolAddress failed on device %d: %s", dev,
+               hipGetErrorString(e));
+    sample_static_ptr[dev] = (float*)p;
+  }
+  *ptr = sample_static_ptr[dev];
+  return 0;
+}
+
+extern "C" int pi_sample_static(int* out, const float* logits, long row_stride, const float* temperature,
+                                const float* uniform, int M, int V, hipStream_t stream) {
+  PI_REQUIRE(M >= 0 && V > 0 && row_stride >= V, "sample_static: bad sizes M=%d V=%d stride=%ld", M, V, row_stride);
+  PI_REQUIRE(temperature == nullptr || uniform != nullptr, "sample_static: temperatures given without uniform numbers");
+  if (M == 0) return 0;
+  const int chunks = pi_sample_chunks(V);
+  if (chunks == 0) return pi_sample(out, logits, row_stride, temperature, uniform, M, V, nullptr, 0, stream);
+  PI_REQUIRE(M <= 65535 && (long)M * chunks * CHUNK_REC <= PI_SAMPLE_STATIC_FLOATS,
+             "sample_static: %d rows of %d logits need %ld floats of chunk records; the library's array holds %d "
+             "(at most %d rows of this length)",
+             M, V, (long)M * chunks * CHUNK_REC, PI_SAMPLE_STATIC_FLOATS, PI_SAMPLE_STATIC_FLOATS / (chunks * CHUNK_REC));
+  float* records = nullptr;
+  if (sample_static_address(&records)) return -1;
+  return pi_sample(out, logits, row_stride, temperature, uniform, M, V, records, PI_SAMPLE_STATIC_FLOATS, stream);
 }

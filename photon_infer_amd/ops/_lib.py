@@ -21,6 +21,7 @@ _SIGNATURES = {
         "pi_paged_attention_general": [P, L, P, L, P, P, I, P, I, P, P, I, I, I, I, I, F, I, L, P],
         "pi_rope_table": [P, P, P, I, I, P],
         "pi_sample": [P, P, L, P, P, I, I, P, L, P],
+        "pi_sample_static": [P, P, L, P, P, I, I, P],
     },
     "bf16": {
         "pi_gemm_mfma": [P, I, L, P, L, P, L, I, I, I, I, P],
