@@ -1,5 +1,5 @@
 """photon_infer_amd: a small, whole LLM inference engine for one AMD MI355X GPU."""
-from .errors import (CacheError, ConfigError, ErrorCode, KernelError, KernelLibraryMissing, OutOfPagesError,
+from .errors import (CacheError, ConfigError, ErrorCode, KernelError, KernelLibraryMissing, OutOfMemoryError, OutOfPagesError,
                      PhotonError, RequestError, UnsupportedModelError, WeightError)
 from .registry import (build_model_spec, get_architecture, load_config, register_architecture,
                        registered_architectures)
@@ -13,7 +13,7 @@ __version__ = "0.1.0"
 __all__ = [
     "ContinuousBatchEngine", "Engine", "EngineOptions", "ModelRunner", "StepEntry", "SamplingParams",
     "write_random_model",
-    "CacheError", "ConfigError", "ErrorCode", "KernelError", "KernelLibraryMissing", "OutOfPagesError",
+    "CacheError", "ConfigError", "ErrorCode", "KernelError", "KernelLibraryMissing", "OutOfMemoryError", "OutOfPagesError",
     "PhotonError", "RequestError", "UnsupportedModelError", "WeightError", "build_model_spec",
     "get_architecture", "load_config", "register_architecture", "registered_architectures",
 ]

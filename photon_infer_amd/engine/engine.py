@@ -46,7 +46,7 @@ class ContinuousBatchEngine:
         self.scheduler = ContinuousBatchScheduler(
             self.runner.cache, options.max_batch, options.max_step_tokens, options.chunk_size,
             self.runner.max_model_len, owner=self.runner)
-        self.sampler = Sampler(self.runner.device)
+        self.sampler = Sampler(self.runner.device, self.runner.workspace)
         self.eos_token_ids = tuple(self.runner.spec.eos_token_ids)
         self.steps = 0
         # a decode step that was launched and whose tokens have not been read yet
@@ -84,6 +84,21 @@ class ContinuousBatchEngine:
 
     def get_stats(self) -> SchedulerStats:
         return self.scheduler.get_stats()
+
+    def abort(self, request_id: int) -> bool:
+        """Cancel a request: waiting, running, or in a decode step that was launched and has not
+        been read yet.  Its slot and pages are free when the call returns (a step already launched
+        may still write the request's last token into them; whatever is given these pages next is
+        launched after it on the same stream), the token of a launched step is dropped, and the
+        request ends with ``finish_reason == "aborted"`` holding what it had generated.  Returns
+        False for a request that is unknown or already finished."""
+        req = self.scheduler.get_request(request_id)
+        if req is None or not self.scheduler.abort(request_id):
+            return False
+        fl = self._in_flight
+        if fl is not None and req in fl.reqs and req not in fl.ended:
+            fl.ended.append(req)          # its row of the launched step is read past, and it is in no later step
+        return True
 
     # ------------------------------------------------------------------ running
     def step(self) -> List[InferenceRequest]:
@@ -172,7 +187,8 @@ class ContinuousBatchEngine:
                  for r in sampled_reqs]
         tokens: List[int] = []
         if self.options.use_graphs and len(sampled_reqs) == len(entries) and all(n == 1 for _, n in batch.items):
-            # single tokens only, every one sampled: the replayed graph (model + sampling kernel)
+            # single tokens only, every one sampled: the replayed graph (model + sampling kernel), or
+            # the same launched one by one when a part of the model does not allow a graph
             if self.options.lookahead:
                 self._launch_decode(sampled_reqs)
                 return []                   # its tokens are read in the next call

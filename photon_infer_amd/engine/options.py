@@ -33,7 +33,9 @@ class EngineOptions:
     dtype: object = "bfloat16"           # compute dtype: "bfloat16" or "float32"
     block_size: int = 16                 # tokens per cache page
     num_blocks: Optional[int] = None     # pages per cache group; None: from max_cache_tokens
-    max_cache_tokens: Optional[int] = None  # tokens the page pool holds; None: max_batch * max_model_len
+    max_cache_tokens: Optional[int] = None  # tokens the page pool holds; None: max_batch * max_model_len, or as many
+                                         # as fit into memory_fraction of the device memory that is free after the weights
+    memory_fraction: float = 0.9         # share of the free device memory that a pool sized by default may take
     max_batch: int = 32                  # most live requests (= state slots)
     max_step_tokens: int = 2048          # token budget of one step
     chunk_size: int = 512                # largest prompt portion of one request in one step (the reference: 256; here a

@@ -172,6 +172,7 @@ class SchedulerStats:
     num_finished: int = 0
     total_requests: int = 0
     num_preemptions: int = 0
+    num_aborted: int = 0
     num_steps: int = 0
     tokens_scheduled: int = 0
 
@@ -195,6 +196,7 @@ class ContinuousBatchScheduler:
         self.requests: Dict[int, InferenceRequest] = {}
         self._next_id = 0
         self._preemptions = 0
+        self._aborted = 0
         self._steps = 0
         self._tokens = 0
 
@@ -318,6 +320,23 @@ class ContinuousBatchScheduler:
         self._steps += 1
         self._tokens += tokens
 
+    def abort(self, request_id: int) -> bool:
+        """Cancel a request wherever it is: a waiting one leaves the queue, a running one gives its
+        slot and pages back at once.  It ends with ``finish_reason = "aborted"`` and keeps what it
+        has generated.  False: unknown or already finished.  (The reference frees only on finish,
+        include/photon/scheduler/continuous_batch_scheduler.hpp:169-182.)"""
+        req = self.requests.get(request_id)
+        if req is None or req.is_finished():
+            return False
+        if req in self.running:
+            self.running.remove(req)
+            self.owner.release(req.request_id)
+        else:
+            self.waiting.remove(req)
+        req.finish("aborted")
+        self._aborted += 1
+        return True
+
     def update_after_step(self, finished: Sequence[InferenceRequest]) -> None:
         """Requests that ended in this step leave the running list and the cache."""
         for req in finished:
@@ -342,7 +361,7 @@ class ContinuousBatchScheduler:
         return SchedulerStats(
             num_running=len(self.running), num_waiting=len(self.waiting),
             num_finished=sum(r.is_finished() for r in self.requests.values()),
-            total_requests=len(self.requests), num_preemptions=self._preemptions,
+            total_requests=len(self.requests), num_preemptions=self._preemptions, num_aborted=self._aborted,
             num_steps=self._steps, tokens_scheduled=self._tokens)
 
     def clear_finished_requests(self) -> None:

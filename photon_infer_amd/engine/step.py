@@ -21,7 +21,7 @@ import torch
 
 from .. import ops
 from ..cache import CacheManager, StateSlots
-from ..errors import CacheError, OutOfPagesError, RequestError
+from ..errors import CacheError, OutOfMemoryError, OutOfPagesError, RequestError
 from ..parts import DecoderModel, LayerCache, ModelSpec, StepContext, plan_cache
 from ..registry import build_model_spec, load_config
 from ..weights import load_model_tensors
@@ -61,7 +61,20 @@ class ModelRunner:
         self.model = DecoderModel(self.spec)
         self.model.load(tensors, self.dtype, self.device)
         del tensors
+        # scratch memory of the kernels and the one residual update that may be pending: this
+        # runner's own, handed to the parts with every step's context
+        self.workspace = ops.KernelWorkspace(self.device)
+        self.workspace.prepare(self.dtype == torch.bfloat16 and ops.fast_kernels_enabled())
         self._build_cache()
+        # what the mixers want planned on the host per step (equal planners are kept once)
+        self.planners = []
+        for e in self.spec.run_order:
+            planner = self.spec.layers[e.layer][1].mixer.step_planner(self.page_size)
+            if planner is not None and planner not in self.planners:
+                self.planners.append(planner)
+        # a decode step is captured as a HIP graph only when every part promises that its launches
+        # do not depend on host-side values of the step
+        self.graph_safe = self.model.graph_safe
         self._graphs: Dict[Tuple[int, int], "_DecodeGraph"] = {}
 
     # ------------------------------------------------------------------ cache set-up
@@ -70,11 +83,36 @@ class ModelRunner:
         self.plan = plan_cache(self.spec)
         self.max_model_len = int(o.max_model_len or self.spec.max_positions)
         self.page_size = int(o.block_size)
-        if o.num_blocks is not None:
-            num_pages = int(o.num_blocks)
+        if self.page_size <= 0 or o.max_batch <= 0:
+            raise RequestError("block_size and max_batch must be positive")
+        # bytes of keys and values that one page holds over all layers that own pages
+        itemsize = torch.empty((), dtype=self.dtype).element_size()
+        page_bytes = sum(2 * nkv * hd * self.page_size * itemsize for g in self.plan.groups for nkv, hd in g.kv_shapes)
+        free, _total = torch.cuda.mem_get_info(self.device)
+        free += torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device)   # torch's own spare blocks
+        if o.num_blocks is not None or o.max_cache_tokens is not None:
+            num_pages = int(o.num_blocks) if o.num_blocks is not None else max(1, -(-int(o.max_cache_tokens) // self.page_size))
+            if num_pages <= 0:
+                raise RequestError("num_blocks / max_cache_tokens must be positive")
+            if num_pages * page_bytes > free:
+                what = f"num_blocks={o.num_blocks}" if o.num_blocks is not None else f"max_cache_tokens={o.max_cache_tokens}"
+                raise OutOfMemoryError(
+                    f"{what} asks for {num_pages} pages of {page_bytes} bytes = {num_pages * page_bytes / 2**30:.1f} GiB of cache; "
+                    f"{free / 2**30:.1f} GiB of device memory are free after the weights "
+                    f"(at most {free // max(1, page_bytes)} pages)")
         else:
-            tokens = o.max_cache_tokens if o.max_cache_tokens is not None else o.max_batch * self.max_model_len
-            num_pages = max(1, -(-int(tokens) // self.page_size))
+            # every slot at full length if that fits; otherwise what the given share of the free
+            # memory holds, and no sequence longer than that
+            wanted = max(1, -(-o.max_batch * self.max_model_len // self.page_size))
+            if not 0.0 < o.memory_fraction <= 1.0:
+                raise RequestError(f"memory_fraction must be in (0, 1], got {o.memory_fraction}")
+            fits = int(free * o.memory_fraction) // max(1, page_bytes) if page_bytes else wanted
+            num_pages = min(wanted, fits)
+            if num_pages < 1:
+                raise OutOfMemoryError(
+                    f"no cache page of {page_bytes} bytes fits into {o.memory_fraction:.2f} of the {free / 2**30:.2f} GiB "
+                    f"of device memory that are free after the weights")
+            self.max_model_len = min(self.max_model_len, num_pages * self.page_size)
         self.num_pages = num_pages
         self.cache = CacheManager([g.window for g in self.plan.groups], self.page_size, num_pages,
                                   o.max_batch, self.max_model_len)
@@ -82,10 +120,14 @@ class ModelRunner:
         # one K and one V pool per run-order entry that owns pages: keys [pages, kv_heads, page,
         # head_dim], values [pages, kv_heads, head_dim, page] (the layout the kernels contract in)
         pools: Dict[int, tuple] = {}
-        for g in self.plan.groups:
-            for entry, (nkv, hd) in zip(g.entries, g.kv_shapes):
-                pools[entry] = (torch.zeros((num_pages, nkv, self.page_size, hd), dtype=self.dtype, device=self.device),
-                                torch.zeros((num_pages, nkv, hd, self.page_size), dtype=self.dtype, device=self.device))
+        try:
+            for g in self.plan.groups:
+                for entry, (nkv, hd) in zip(g.entries, g.kv_shapes):
+                    pools[entry] = (torch.zeros((num_pages, nkv, self.page_size, hd), dtype=self.dtype, device=self.device),
+                                    torch.zeros((num_pages, nkv, hd, self.page_size), dtype=self.dtype, device=self.device))
+        except torch.OutOfMemoryError as e:
+            pools.clear()
+            raise OutOfMemoryError(f"the cache pools ({num_pages} pages of {page_bytes} bytes) do not fit the device: {e}") from None
         self.layer_caches: List[LayerCache] = []
         for i, e in enumerate(self.spec.run_order):
             owner = i if e.cache_of is None else e.cache_of
@@ -155,9 +197,14 @@ class ModelRunner:
         }
         for g in range(len(cache.groups)):
             parts[f"table{g}"] = np.ascontiguousarray(cache.table_rows(g, slots, width)).reshape(-1)
-        extra = ops.plan_attention(q_lens, kv_lens, self.dtype) if T else {}
-        parts.update(extra.get("arrays", {}))
-        views = _upload(parts, self.device)
+        planned = []
+        for i, planner in enumerate(self.planners):
+            made = planner.plan(q_lens, kv_lens)
+            if made is not None:
+                arrays, finish = made
+                parts.update({f"plan{i}.{name}": arr for name, arr in arrays.items()})
+                planned.append((planner, f"plan{i}.", tuple(arrays), finish))
+        views = ops.upload_arrays(parts, self.device)
         ctx = StepContext(
             T=T, R=R, dtype=self.dtype,
             token_ids=views["token_ids"], positions=views["positions"], req_of_token=views["req_of_token"],
@@ -165,9 +212,10 @@ class ModelRunner:
             block_tables={g: views[f"table{g}"].view(R, width) for g in range(len(cache.groups))},
             logit_rows=views["logit_rows"],
             q_lens=q_lens, kv_lens=kv_lens, max_q_len=max(q_lens), max_kv_len=max(kv_lens),
-            all_decode=all(n == 1 for n in q_lens), host_slots=slots,
+            all_decode=all(n == 1 for n in q_lens), host_slots=slots, workspace=self.workspace,
         )
-        ops.attach_attention_plan(ctx, extra, views)
+        for planner, prefix, names, finish in planned:
+            ctx.plans[planner] = finish({name: views[prefix + name] for name in names})
         return ctx
 
     def _reserve(self, entries: Sequence[StepEntry]) -> List[int]:
@@ -208,9 +256,10 @@ class ModelRunner:
                     feed: Optional[Tuple[torch.Tensor, Sequence[int]]] = None) -> torch.Tensor:
         """A batch of single tokens, one per request, each wanting its next token: the model
         and the sampling kernel run as one replayed HIP graph (captured per batch size and
-        length bucket at first use).  Returns the chosen token ids (int32 [R], on the device);
-        the same buffer is written by the next step of the same shape, so read or copy it
-        before launching that one.
+        length bucket at first use) - or, when a part of the model does not promise that its
+        launches are the same from step to step (``Part.graph_safe``), eagerly with the same
+        kernels.  Returns the chosen token ids (int32 [R], on the device); the same buffer is
+        written by the next step of the same shape, so read or copy it before launching that one.
 
         ``feed`` = (ids, rows): the tokens are not known on the host yet; request i's token is
         ``ids[rows[i]]``, taken on the device (``ids``: what an earlier decode_step returned).
@@ -223,6 +272,8 @@ class ModelRunner:
                 raise RequestError("decode_step: one fed row per request is needed")
             entries = [StepEntry(e.rid, [0], e.want) for e in entries]     # placeholders pass the vocabulary check
         self._check(entries)
+        if not (self.graph_safe and self.options.use_graphs):
+            return self._decode_eager(entries, temperatures, uniforms, feed)
         slots = self._reserve(entries)
         lengths = self.cache.lengths_of(slots)
         # one graph per batch size and length bucket: the attention kernel's key ranges follow the bucket
@@ -235,18 +286,22 @@ class ModelRunner:
         return out
 
 
-def _upload(parts: Dict[str, np.ndarray], device) -> Dict[str, torch.Tensor]:
-    """Concatenate int32 arrays (each padded to 16 bytes), copy once, return device views."""
-    offsets, total = {}, 0
-    for name, arr in parts.items():
-        offsets[name] = (total, arr.size)
-        total += (arr.size + 3) // 4 * 4
-    packed = np.zeros(max(total, 4), np.int32)
-    for name, arr in parts.items():
-        o, n = offsets[name]
-        packed[o:o + n] = arr
-    dev = torch.from_numpy(packed).to(device)
-    return {name: dev[o:o + n] for name, (o, n) in offsets.items()}
+    def _decode_eager(self, entries, temperatures, uniforms, feed) -> torch.Tensor:
+        """``decode_step`` without a graph: the step function and the sampling kernel, launched
+        one by one.  Parts may read the step's shape and slots on the host."""
+        R = len(entries)
+        entries = [StepEntry(e.rid, e.tokens, [0]) for e in entries]
+        slots = self._reserve(entries)
+        ctx = self.build_context(entries)
+        if feed is not None:      # the tokens come from an earlier step's result, on the device
+            rows = torch.tensor(list(feed[1]), dtype=torch.int32).to(self.device)
+            torch.index_select(feed[0], 0, rows, out=ctx.token_ids)
+        logits = self.model.forward(ctx, self.layer_caches)
+        params = torch.from_numpy(np.asarray([list(temperatures), list(uniforms)], np.float32)).to(self.device)
+        out = torch.empty(R, dtype=torch.int32, device=self.device)   # a buffer of its own: the step before may still be unread
+        ops.sample(out, logits, params[0], params[1], ws=self.workspace)
+        self.cache.commit_step(slots, [1] * R)
+        return out
 
 
 class _DecodeGraph:
@@ -294,7 +349,8 @@ class _DecodeGraph:
             T=R, R=R, dtype=runner.dtype, token_ids=d["token_ids"], positions=d["positions"],
             req_of_token=d["req_of_token"], q_start=d["q_start"], kv_len=d["kv_len"], slots=d["slots"],
             block_tables={g: d[f"table{g}"].view(R, self.width) for g in range(G)}, logit_rows=d["logit_rows"],
-            q_lens=[1] * R, kv_lens=(), max_q_len=1, max_kv_len=length_bucket, all_decode=True)
+            q_lens=[1] * R, kv_lens=(), max_q_len=1, max_kv_len=length_bucket, all_decode=True,
+            workspace=runner.workspace)
         self.feed_rows = d["feed_rows"]
         self.temps = d["temps"].view(torch.float32)
         self.uniforms = d["uniforms"].view(torch.float32)
@@ -325,7 +381,7 @@ class _DecodeGraph:
 
     def _body(self) -> None:
         logits = self.runner.model.forward(self.ctx, self.runner.layer_caches)
-        ops.sample(self.sampled, logits, self.temps, self.uniforms)
+        ops.sample(self.sampled, logits, self.temps, self.uniforms, ws=self.runner.workspace)
 
     def run(self, entries, slots, lengths, temperatures, uniforms, feed=None) -> torch.Tensor:
         self._fill(entries, slots, lengths, temperatures, uniforms, feed)

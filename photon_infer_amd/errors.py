@@ -89,6 +89,12 @@ class OutOfPagesError(PhotonError):
     code = ErrorCode.OUT_OF_MEMORY
 
 
+class OutOfMemoryError(PhotonError):
+    """Device memory cannot hold what was asked for (the cache pools, a workspace)."""
+
+    code = ErrorCode.OUT_OF_MEMORY
+
+
 class CacheError(PhotonError):
     """Misuse of the cache manager: double free, unknown request, no free slot."""
 

@@ -17,6 +17,7 @@ import torch
 
 from ..errors import KernelError
 from . import _lib
+from .workspace import KernelWorkspace, Partials
 
 PI_F32, PI_BF16 = 0, 1
 MAX_HEAD_DIM = 256
@@ -102,8 +103,10 @@ def embedding(out: torch.Tensor, table: torch.Tensor, ids: torch.Tensor) -> None
 
 
 def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float,
-            rows: Optional[torch.Tensor] = None) -> None:
-    """out[m, :] = weight * x[r, :] / sqrt(mean(x[r, :]^2) + eps), r = rows[m] (or m)."""
+            rows: Optional[torch.Tensor] = None, ws: Optional[KernelWorkspace] = None) -> None:
+    """out[m, :] = weight * x[r, :] / sqrt(mean(x[r, :]^2) + eps), r = rows[m] (or m).  An update of
+    ``x`` that is still pending in ``ws`` is added first, in the same pass, and written back to
+    ``x`` (with ``rows``: to those rows only; the others are not read again by this caller)."""
     _gpu(out, x, weight, rows)
     M, D = out.shape
     if x.dtype != torch.float32 or not x.is_contiguous() or x.dim() != 2 or x.shape[1] != D:
@@ -115,7 +118,9 @@ def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float
             raise KernelError(f"rmsnorm: {x.shape[0]} input rows for {M} output rows")
     else:
         _i32(rows, "rmsnorm rows", M)
-    pending = _take_deferred(x)
+    pending = ws.take_pending(x) if ws is not None else None
+    if pending is not None:
+        ws.counts["added_by_norm"] += 1
     part, splits = (pending.part.data_ptr(), pending.splits) if pending is not None else (None, 0)
     _lib.call("core", "pi_rmsnorm", out.data_ptr(), _dt(out), x.data_ptr(), _ptr(rows), weight.data_ptr(),
               _dt(weight), float(eps), M, D, part, splits, x.shape[0], _stream())
@@ -123,39 +128,32 @@ def rmsnorm(out: torch.Tensor, x: torch.Tensor, weight: torch.Tensor, eps: float
 
 # ----------------------------------------------------------------------------- deferred updates
 # A product into the residual stream whose k-range was split over blocks may stay in pieces
-# (a `Partials`) until the next reader of the stream: ``rmsnorm`` folds the sum of the pieces
-# and the residual add into its own pass.  Whoever reads the stream in any other way calls
-# ``materialize`` first.  Only callers that pass ``may_defer=True`` to ``gemm`` ever leave an
-# update pending, and a block arrangement must materialize before it hands the stream to a
-# part that does not read it through ``rmsnorm``.
-def _take_deferred(x: torch.Tensor):
-    from . import fast
-    p = fast.PENDING.pop(x.data_ptr(), None)
-    if p is not None and (p.M, p.N) != tuple(x.shape):
-        fast.reduce_into(x, p, accumulate=True)      # not the tensor it was made for: play safe
-        return None
-    return p
-
-
-def materialize(x: torch.Tensor) -> torch.Tensor:
-    """Apply an update of ``x`` that is still pending, if there is one."""
-    from . import fast
-    p = fast.PENDING.pop(x.data_ptr(), None)
+# (``Partials`` in the caller's ``KernelWorkspace``) until the next reader of the stream:
+# ``rmsnorm`` folds the sum of the pieces and the residual add into its own pass.  Whoever reads
+# the stream in any other way calls ``materialize`` first.  Only callers that pass
+# ``may_defer=True`` and a workspace to ``gemm`` ever leave an update pending (one at most per
+# workspace), and a block arrangement must materialize before it hands the stream to a part that
+# does not read it through ``rmsnorm``.
+def materialize(x: torch.Tensor, ws: Optional[KernelWorkspace]) -> torch.Tensor:
+    """Apply an update of ``x`` that is still pending in ``ws``, if there is one."""
+    p = ws.take_pending(x) if ws is not None else None
     if p is not None:
+        from . import fast
         fast.reduce_into(x, p, accumulate=True)
+        ws.counts["applied"] += 1
     return x
 
 
-def reset_deferred() -> None:
-    """Forget every pending update (start of a step)."""
-    from . import fast
-    fast.PENDING.clear()
+def reset_deferred(ws: Optional[KernelWorkspace]) -> None:
+    """Forget a pending update (start of a step: nothing of an earlier, failed step may linger)."""
+    if ws is not None:
+        ws.pending = None
 
 
-def discard_deferred(x: torch.Tensor) -> None:
+def discard_deferred(x: torch.Tensor, ws: Optional[KernelWorkspace]) -> None:
     """Forget a pending update of ``x`` (the stream is not read again)."""
-    from . import fast
-    fast.PENDING.pop(x.data_ptr(), None)
+    if ws is not None and ws.take_pending(x) is not None:
+        ws.counts["discarded"] += 1
 
 
 def swiglu(out: torch.Tensor, gate_up: torch.Tensor, block: int = 0) -> None:
@@ -170,7 +168,8 @@ def swiglu(out: torch.Tensor, gate_up: torch.Tensor, block: int = 0) -> None:
     _lib.call("core", "pi_swiglu", out.data_ptr(), gate_up.data_ptr(), _dt(out), T, I, int(block), _stream())
 
 
-def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate_up: torch.Tensor, block: int = 0) -> None:
+def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate_up: torch.Tensor, block: int = 0,
+                ws: Optional[KernelWorkspace] = None) -> None:
     """out[M, I] = silu(a @ Wg^T) * (a @ Wu^T) where ``w_gate_up`` [2I, K] holds the gate and
     up rows in halves (``block`` 0) or interleaved in blocks of ``block`` rows.  With bfloat16
     operands and blocks of 16 the product and the activation are one kernel."""
@@ -185,16 +184,18 @@ def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate_up: torch.Tensor, blo
         if fast.gemm_swiglu(out, a, w_gate_up, M, 2 * I, a.shape[1], _rows(a, "gemm a"), _rows(w_gate_up, "gemm w")):
             return
     gu = torch.empty((M, 2 * I), dtype=a.dtype, device=a.device)
-    gemm(gu, a, w_gate_up)
+    gemm(gu, a, w_gate_up, ws=ws)
     swiglu(out, gu, block)
 
 
 def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, accumulate: bool = False,
-         may_defer: bool = False) -> None:
+         may_defer: bool = False, ws: Optional[KernelWorkspace] = None) -> None:
     """out[M, N] (+)= a[M, K] @ w[N, K]^T with float32 accumulation.
 
-    ``may_defer`` (with ``accumulate``): the caller promises that ``out`` is next read by
-    ``rmsnorm`` or ``materialize``; a product that was split over k may then stay in pieces."""
+    ``ws``: where a product split over k keeps its pieces (without one, memory of this call's own).
+    ``may_defer`` (with ``accumulate`` and ``ws``): the caller promises that ``out`` is next read
+    by ``rmsnorm`` or ``materialize`` with the same workspace; a product that was split over k may
+    then stay in pieces there."""
     _gpu(out, a, w)
     if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
         raise KernelError("gemm: operands must be 2-D")
@@ -208,10 +209,10 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, accumulate: bool =
     if M == 0:
         return
     if accumulate:
-        materialize(out)
+        materialize(out, ws)
     if _FAST and a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16:
         from . import fast
-        if fast.gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc, may_defer and accumulate and out.is_contiguous()):
+        if fast.gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc, may_defer and accumulate and out.is_contiguous(), ws):
             return
     _lib.call("core", "pi_gemm_general", out.data_ptr(), _dt(out), ldc, a.data_ptr(), _dt(a), lda, w.data_ptr(),
               _dt(w), ldw, M, N, K, int(accumulate), _stream())
@@ -255,17 +256,19 @@ def _rotary_args(rotary, positions, T):
     return table.data_ptr(), rdim, inter, table
 
 
-def qkv_projection(h: torch.Tensor, w_qkv: torch.Tensor, dtype: torch.dtype):
+def qkv_projection(h: torch.Tensor, w_qkv: torch.Tensor, dtype: torch.dtype, ws: Optional[KernelWorkspace] = None):
     """h @ w_qkv^T for the attention mixer: a tensor [T, N] in ``dtype``, or - when the
-    product was split over k - its pieces (``fast.Partials``), which ``rope_kv_write`` sums
-    on the fly so that the rotation sees float32 values."""
-    if _FAST and h.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and h.is_cuda:
+    product was split over k and there is a workspace to keep them in - its pieces
+    (``Partials``), which ``rope_kv_write`` sums on the fly so that the rotation sees float32
+    values.  The pieces are good until the next product with the same workspace."""
+    if _FAST and ws is not None and h.dtype == torch.bfloat16 and w_qkv.dtype == torch.bfloat16 and h.is_cuda:
         from . import fast
-        p = fast.gemm_pieces(h, w_qkv)
+        p = fast.gemm_pieces(h, w_qkv, ws)
         if p is not None:
+            ws.counts["qkv_pieces"] += 1
             return p
     out = torch.empty((h.shape[0], w_qkv.shape[0]), dtype=dtype, device=h.device)
-    gemm(out, h, w_qkv)
+    gemm(out, h, w_qkv, ws=ws)
     return out
 
 
@@ -325,7 +328,7 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
 def decode_attention_from_projection(out: torch.Tensor, qkv, ctx, rotary, num_heads: int, num_kv_heads: int,
                                      head_dim: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
                                      block_table: torch.Tensor, page_size: int, scale: float, window: int,
-                                     write_kv: bool) -> bool:
+                                     write_kv: bool, ws: Optional[KernelWorkspace] = None) -> bool:
     """For a step that holds single tokens only: rotation, cache write and attention in one
     kernel, from the q|k|v projection ``qkv`` (a tensor [T, N] or ``fast.Partials``, columns
     [q heads | k heads | v heads]).  Returns False, having done nothing, when the step, the
@@ -334,7 +337,7 @@ def decode_attention_from_projection(out: torch.Tensor, qkv, ctx, rotary, num_he
     if not (_FAST and out.dtype == torch.bfloat16 and out.is_cuda and getattr(ctx, "all_decode", False)):
         return False
     from . import fast
-    if not isinstance(qkv, fast.Partials) and qkv.dtype != torch.bfloat16:
+    if not isinstance(qkv, Partials) and qkv.dtype != torch.bfloat16:
         return False
     T = out.shape[0]
     table = None
@@ -350,16 +353,17 @@ def decode_attention_from_projection(out: torch.Tensor, qkv, ctx, rotary, num_he
     if block_table.dim() != 2 or block_table.dtype != torch.int32 or not block_table.is_contiguous():
         raise KernelError("attention: block table must be contiguous int32 [requests, width]")
     return fast.decode_attention_from_projection(out, qkv, ctx, table, num_heads, num_kv_heads, head_dim, k_cache, v_cache,
-                                                 block_table, page_size, scale, window, pages, write_kv)
+                                                 block_table, page_size, scale, window, pages, write_kv, ws)
 
 
 def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                     block_table: torch.Tensor, ctx, num_heads: int, num_kv_heads: int, head_dim: int,
-                    page_size: int, scale: float, window: int = 0) -> None:
+                    page_size: int, scale: float, window: int = 0, ws: Optional[KernelWorkspace] = None) -> None:
     """Causal attention of every token of the step over its request's pages.
 
-    ``ctx`` carries ``positions`` and ``req_of_token`` ([T] int32) and, for the
-    matrix-core kernels, the work lists the step function made.
+    ``ctx`` carries ``positions`` and ``req_of_token`` ([T] int32), the step's shape on the host
+    (``q_lens``, ``kv_lens``, ``all_decode``) and, in ``plans``, the work lists that the
+    matrix-core kernels want (made here when the step function has not).
     """
     _gpu(out, q, k_cache, v_cache, block_table, ctx.positions, ctx.req_of_token)
     T = q.shape[0]
@@ -376,7 +380,7 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
     if _FAST and q.dtype == torch.bfloat16:
         from . import fast
         if fast.paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
-                                page_size, scale, window, pages):
+                                page_size, scale, window, pages, ws):
             return
     _lib.call("core", "pi_paged_attention_general", out.data_ptr(), _rows(out, "attention out"), q.data_ptr(),
               _rows(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), _dt(q), block_table.data_ptr(),
@@ -385,7 +389,7 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
 
 
 def sample(out: torch.Tensor, logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,
-           uniform: Optional[torch.Tensor] = None) -> None:
+           uniform: Optional[torch.Tensor] = None, ws: Optional[KernelWorkspace] = None) -> None:
     """out[m] = argmax of row m (lowest index among equals) where temperature[m] <= 0 or
     no temperatures are given; otherwise the first index whose cumulative
     softmax(logits / temperature) reaches uniform[m]."""
@@ -399,14 +403,15 @@ def sample(out: torch.Tensor, logits: torch.Tensor, temperature: Optional[torch.
             raise KernelError(f"sample: {what} must be contiguous float32 [{M}]")
     if temperature is not None and uniform is None:
         raise KernelError("sample: temperatures given without uniform numbers")
-    ws = _SAMPLE_WS.get(logits.device)
-    if ws is None:
-        ws = _SAMPLE_WS[logits.device] = torch.empty(1 << 18, dtype=torch.float32, device=logits.device)
+    chunks = _lib.load("core").pi_sample_chunks(V)
+    if chunks == 0:
+        part = None
+    elif ws is not None:
+        part = ws.sample_part
+    else:
+        part = torch.empty(M * chunks * 4, dtype=torch.float32, device=logits.device)
     _lib.call("core", "pi_sample", out.data_ptr(), logits.data_ptr(), _rows(logits, "logits"), _ptr(temperature),
-              _ptr(uniform), M, V, ws.data_ptr(), ws.numel(), _stream())
-
-
-_SAMPLE_WS: dict = {}
+              _ptr(uniform), M, V, _ptr(part), 0 if part is None else part.numel(), _stream())
 
 
 # ----------------------------------------------------------------------------- work lists
@@ -416,16 +421,17 @@ def decode_length_bucket(max_kv_len: int) -> int:
     return fast.decode_length_bucket(max_kv_len)
 
 
-def plan_attention(q_lens, kv_lens, dtype) -> dict:
-    """Host-side work lists (int32 arrays to upload with the step's metadata) that the
-    matrix-core attention kernels want; empty for the general kernels."""
-    if _FAST and dtype == torch.bfloat16:
+def attention_planner(dtype: torch.dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int,
+                      window: int, device):
+    """What makes a step's work lists for an attention mixer of these sizes (a hashable object with
+    ``plan(q_lens, kv_lens)``; equal ones share a plan), or None when its kernels need none."""
+    if _FAST and dtype == torch.bfloat16 and _lib.build.MODULES["bf16"]:
         from . import fast
-        return fast.plan_attention(q_lens, kv_lens)
-    return {}
+        return fast.attention_planner(dtype, num_heads, num_kv_heads, head_dim, page_size, int(window), torch.device(device))
+    return None
 
 
-def attach_attention_plan(ctx, plan: dict, views: dict) -> None:
-    if plan:
-        from . import fast
-        fast.attach_attention_plan(ctx, plan, views)
+def upload_arrays(arrays, device):
+    """int32 host arrays by name -> device views of one packed copy."""
+    from . import fast
+    return fast.upload_arrays(arrays, device)

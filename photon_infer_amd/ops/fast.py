@@ -14,13 +14,15 @@ Which kernel takes what:
 from __future__ import annotations
 
 import ctypes
+import functools
 from dataclasses import dataclass
-from typing import Dict, List, Optional
+from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
 from . import _lib
+from .workspace import GEMM_PART_FLOATS, KernelWorkspace, Partials, PendingUpdate
 
 EPI_BF16, EPI_F32, EPI_ACCUM, EPI_SWIGLU = 0, 1, 2, 3
 SKINNY_MAX_ROWS = 128          # up to this many tokens the weight-streaming kernels serve a product (measured against the tile kernel)
@@ -29,56 +31,11 @@ TARGET_BLOCKS = 512            # blocks wanted in flight to keep HBM busy
 SHARED_FROM_TOKENS = 32        # more tokens than this: the skinny kernel that shares activations per block ...
 SHARED_ROWS_PER_BLOCK = 64     # ... with this many weight rows per block ...
 SHARED_TARGET_BLOCKS = 256     # ... and this many blocks wanted (one per compute unit)
-GEMM_PART_FLOATS = 16 << 20    # workspace for the pieces of products split over k (64 MB)
 TILE_MAX_SPLITS = 4
 PIECES_BELOW_TILES = 200       # fewer 128 x 128 tiles than this: q, k, v of a prompt portion are left in k pieces too
-ATTN_PART_FLOATS = 4 << 20     # key-split partial results of decode attention
 MAX_DECODE_SPLITS = 64         # the combine kernel holds one key range per lane
 DECODE_WAVES_WANTED = 512      # waves of the decode attention kernel that fill the chip (measured at batch 1 to 64: more is never faster)
 DECODE_MIN_KEYS_PER_SPLIT = 128
-
-
-class _Workspace:
-    """Scratch the kernels share on one device: the pieces of products split over k and of
-    attention split over keys.  Kernels on one stream run one after another, so one set is
-    enough; a product left in pieces (see ``Partials``) owns the product scratch until it is
-    consumed."""
-
-    def __init__(self, device):
-        self.gemm_part = torch.empty(GEMM_PART_FLOATS, dtype=torch.float32, device=device)
-        self.attn_part = torch.empty(ATTN_PART_FLOATS, dtype=torch.float32, device=device)
-        self.tile_part = torch.empty(4, dtype=torch.float32, device=device)   # partial results of cut tiles, grown on demand
-        self.device = device
-        self.splits_out = ctypes.c_int(0)
-
-    def tile_part_for(self, floats: int) -> torch.Tensor:
-        if self.tile_part.numel() < floats:
-            self.tile_part = torch.empty(floats, dtype=torch.float32, device=self.device)
-        return self.tile_part
-
-
-@dataclass
-class Partials:
-    """A product [M, N] whose k-range was split: ``part`` holds float32 [splits, M, N]."""
-
-    part: torch.Tensor
-    splits: int
-    M: int
-    N: int
-
-
-# updates of a residual stream that are still in pieces, keyed by the stream's address
-PENDING: Dict[int, Partials] = {}
-
-
-_WORKSPACES: Dict[torch.device, _Workspace] = {}
-
-
-def workspace(device) -> _Workspace:
-    ws = _WORKSPACES.get(device)
-    if ws is None:
-        ws = _WORKSPACES[device] = _Workspace(device)
-    return ws
 
 
 def _stream() -> int:
@@ -109,22 +66,47 @@ def _tile_splits(M: int, N: int, K: int) -> int:
     return max(1, splits)
 
 
-def _flush_pending() -> None:
-    """The product scratch is about to be reused: finish whatever still lives in it."""
-    for ptr in list(PENDING):
-        p = PENDING.pop(ptr)
-        _lib.call("bf16", "pi_splitk_reduce", ptr, EPI_ACCUM, p.N, p.part.data_ptr(), p.splits, p.M, p.N, _stream())
+def flush(ws: Optional[KernelWorkspace]) -> None:
+    """The product scratch is about to be reused: apply the update that still lives in it."""
+    if ws is None or ws.pending is None:
+        return
+    p, ws.pending = ws.pending, None
+    reduce_into(p.target, p.pieces, accumulate=True)
+    ws.counts["flushed"] += 1
 
 
-def _skinny(out_ptr: int, epilogue: int, ldc: int, a, w, M, N, K, lda, ldw, splits: int) -> Optional[Partials]:
+def _piece_buffer(ws: Optional[KernelWorkspace], floats: int, device) -> torch.Tensor:
+    """Where the pieces of a split product go: the workspace's buffer (whose last tenant is
+    applied first), or memory of this call's own."""
+    if ws is None:
+        return torch.empty(floats, dtype=torch.float32, device=device)
+    flush(ws)
+    return ws.gemm_part
+
+
+def _skinny(out_ptr: int, epilogue: int, ldc: int, a, w, M, N, K, lda, ldw, splits: int,
+            ws: Optional[KernelWorkspace]) -> Optional[Partials]:
     """Run the weight-streaming kernel; returns the pieces when the product was split."""
-    ws = workspace(a.device)
-    if splits > 1:
-        _flush_pending()
+    buf = _piece_buffer(ws, splits * M * N, a.device) if splits > 1 else None
+    made = ctypes.c_int(0)
     _lib.call("bf16", "pi_gemm_skinny", out_ptr, epilogue, ldc, a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K, splits,
-              ws.gemm_part.data_ptr(), ws.gemm_part.numel(), ctypes.byref(ws.splits_out), _stream())
-    made = ws.splits_out.value
-    return Partials(ws.gemm_part, made, M, N) if made > 1 else None
+              None if buf is None else buf.data_ptr(), 0 if buf is None else buf.numel(), ctypes.byref(made), _stream())
+    if made.value > 1:
+        if ws is not None:
+            ws.counts["split_products"] += 1
+        return Partials(buf, made.value, M, N)
+    return None
+
+
+def _tiles_in_pieces(a, w, M, N, K, lda, ldw, splits: int, ws: Optional[KernelWorkspace]) -> Optional[Partials]:
+    """The tile kernel with its k-range split: float32 pieces, nothing else written."""
+    buf = _piece_buffer(ws, splits * M * N, a.device)
+    made = _lib.load("bf16").pi_gemm_mfma_pieces(K, splits)
+    _lib.call("bf16", "pi_gemm_mfma", buf.data_ptr(), EPI_F32, N, a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K, splits,
+              _stream())
+    if ws is not None:
+        ws.counts["split_products"] += 1
+    return Partials(buf, made, M, N)
 
 
 def reduce_into(out: torch.Tensor, p: Partials, accumulate: bool) -> None:
@@ -133,7 +115,7 @@ def reduce_into(out: torch.Tensor, p: Partials, accumulate: bool) -> None:
               _stream())
 
 
-def gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc, may_defer=False) -> bool:
+def gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc, may_defer=False, ws: Optional[KernelWorkspace] = None) -> bool:
     if not _gemm_ok(a, w, K, lda, ldw):
         return False
     if accumulate:
@@ -144,33 +126,33 @@ def gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc, may_defer=False) -> bool
         epilogue = EPI_F32
     else:
         return False
+    may_defer = may_defer and ws is not None      # pieces can only wait in a workspace that outlives the call
     if M > SKINNY_MAX_ROWS:
+        # few output tiles, long k: split k so that every compute unit has work; the pieces
+        # stay in the workspace for the next norm of this stream
         splits = _tile_splits(M, N, K) if may_defer else 1
         if splits > 1:
-            # few output tiles, long k: split k so that every compute unit has work; the pieces
-            # stay in the workspace for the next norm of this stream
-            ws = workspace(a.device)
-            _flush_pending()
-            made = _lib.load("bf16").pi_gemm_mfma_pieces(K, splits)
-            _lib.call("bf16", "pi_gemm_mfma", ws.gemm_part.data_ptr(), EPI_F32, N, a.data_ptr(), lda, w.data_ptr(), ldw,
-                      M, N, K, splits, _stream())
-            PENDING[out.data_ptr()] = Partials(ws.gemm_part, made, M, N)
+            ws.pending = PendingUpdate(out, _tiles_in_pieces(a, w, M, N, K, lda, ldw, splits, ws))
+            ws.counts["deferred"] += 1
             return True
         _lib.call("bf16", "pi_gemm_mfma", out.data_ptr(), epilogue, ldc, a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K, 1,
                   _stream())
         return True
-    pieces = _skinny(out.data_ptr(), epilogue, ldc, a, w, M, N, K, lda, ldw, _skinny_splits(M, N, K))
+    pieces = _skinny(out.data_ptr(), epilogue, ldc, a, w, M, N, K, lda, ldw, _skinny_splits(M, N, K), ws)
     if pieces is not None:
         if may_defer:
-            PENDING[out.data_ptr()] = pieces          # the next norm of this stream adds them
+            ws.pending = PendingUpdate(out, pieces)          # the next norm of this stream adds them
+            ws.counts["deferred"] += 1
         else:
             _lib.call("bf16", "pi_splitk_reduce", out.data_ptr(), epilogue, ldc, pieces.part.data_ptr(), pieces.splits,
                       M, N, _stream())
     return True
 
 
-def gemm_pieces(a, w) -> Optional[Partials]:
-    """a @ w^T left in pieces, if this product is one the weight-streaming kernel would split."""
+def gemm_pieces(a, w, ws: Optional[KernelWorkspace]) -> Optional[Partials]:
+    """a @ w^T left in pieces in the workspace, if this product is one whose k-range is split."""
+    if ws is None:
+        return None
     M, K = a.shape
     N = w.shape[0]
     lda, ldw = a.stride(0) if M > 1 else K, w.stride(0)
@@ -183,16 +165,12 @@ def gemm_pieces(a, w) -> Optional[Partials]:
         splits = _tile_splits(M, N, K) if tiles < PIECES_BELOW_TILES else 1
         if splits <= 1:
             return None
-        ws = workspace(a.device)
-        _flush_pending()
-        made = _lib.load("bf16").pi_gemm_mfma_pieces(K, splits)
-        _lib.call("bf16", "pi_gemm_mfma", ws.gemm_part.data_ptr(), EPI_F32, N, a.data_ptr(), lda, w.data_ptr(), ldw,
-                  M, N, K, splits, _stream())
-        return Partials(ws.gemm_part, made, M, N) if made > 1 else None
+        p = _tiles_in_pieces(a, w, M, N, K, lda, ldw, splits, ws)
+        return p if p.splits > 1 else None
     splits = _skinny_splits(M, N, K)
     if splits <= 1:
         return None
-    return _skinny(0, EPI_F32, N, a, w, M, N, K, lda, ldw, splits)
+    return _skinny(0, EPI_F32, N, a, w, M, N, K, lda, ldw, splits, ws)
 
 
 def gemm_swiglu(out, a, w, M, N, K, lda, ldw) -> bool:
@@ -203,7 +181,7 @@ def gemm_swiglu(out, a, w, M, N, K, lda, ldw) -> bool:
         _lib.call("bf16", "pi_gemm_mfma", out.data_ptr(), EPI_SWIGLU, out.stride(0), a.data_ptr(), lda, w.data_ptr(), ldw,
                   M, N, K, 1, _stream())
     else:
-        _skinny(out.data_ptr(), EPI_SWIGLU, out.stride(0), a, w, M, N, K, lda, ldw, 1)
+        _skinny(out.data_ptr(), EPI_SWIGLU, out.stride(0), a, w, M, N, K, lda, ldw, 1, None)
     return True
 
 
@@ -229,24 +207,31 @@ def deal_tiles(walks: List[int], seats: int) -> np.ndarray:
     return order
 
 
-def _tiles(ctx, tile_rows: int, window: int, num_kv_heads: int, device, skip=()):
-    """Work list of the tile kernel: (request, first token) of every tile and their deal to the
-    blocks; cached on the step (layers with the same window share it).  ``skip``: requests
-    that another kernel serves."""
-    cache = getattr(ctx, "_attention_tiles", None)
-    if cache is None:
-        cache = {}
-        try:
-            ctx._attention_tiles = cache
-        except AttributeError:
-            pass
-    key = (tile_rows, window, num_kv_heads, bool(skip))
-    hit = cache.get(key)
-    if hit is None:
+@dataclass(frozen=True)
+class AttentionPlanner:
+    """Makes a step's work lists for the prompt-attention tile kernel.  Mixers whose planners are
+    equal (same tile height, window, kv heads) share one plan per step.  ``plan`` runs on the
+    host before the step's metadata is uploaded; its arrays ride in that one copy."""
+
+    tile_rows: int            # query rows of a tile (the kernel's, for these head counts)
+    window: int               # 0: all keys
+    num_kv_heads: int
+    singles_apart: bool       # requests that bring one token go to the key-split kernel instead
+    units: int                # compute units of the device
+
+    def plan(self, q_lens: Sequence[int], kv_lens: Sequence[int]):
+        """None for a step of single tokens only (the key-split kernel needs no list); otherwise
+        (int32 host arrays by name, a function from their device views to a ``TilePlan``)."""
+        if self.singles_apart and all(n == 1 for n in q_lens):
+            return None
+        tile_rows, window = self.tile_rows, self.window
+        singles = tuple(r for r, n in enumerate(q_lens) if n == 1) if self.singles_apart else ()
+        if len(singles) == len(q_lens):
+            singles = ()
+        skipped = set(singles)
         req, q0, walks, first_row, n_tok = [], [], [], [], []
-        skipped = set(skip)
         row0 = 0
-        for r, (n, kv) in enumerate(zip(ctx.q_lens, ctx.kv_lens)):
+        for r, (n, kv) in enumerate(zip(q_lens, kv_lens)):
             if r not in skipped:
                 for start in range(0, n, tile_rows):
                     req.append(r)
@@ -258,8 +243,7 @@ def _tiles(ctx, tile_rows: int, window: int, num_kv_heads: int, device, skip=())
                     first_row.append(row0 + start)
                     n_tok.append(min(tile_rows, n - start))
             row0 += n
-        units = torch.cuda.get_device_properties(device).multi_processor_count
-        seats_wanted = max(1, ATTENTION_BLOCKS_PER_UNIT * units // max(1, num_kv_heads))
+        seats_wanted = max(1, ATTENTION_BLOCKS_PER_UNIT * self.units // max(1, self.num_kv_heads))
         # too few tiles for the chip (a portion of a few hundred tokens): cut the key range of
         # the long ones into equal shares; the shares' partial results are merged afterwards
         cuts = cut_count(walks, seats_wanted)
@@ -274,15 +258,58 @@ def _tiles(ctx, tile_rows: int, window: int, num_kv_heads: int, device, skip=())
                 t_walk.append(-(-walks[i] // k))
         seats = max(1, min(len(t_req), seats_wanted))
         order = deal_tiles(t_walk, seats)
-        n = len(t_req)
-        host = np.concatenate([np.asarray(t_req, np.int32), np.asarray(t_q0, np.int32), np.asarray(t_cut, np.int32),
-                               np.asarray(t_z0, np.int32), np.asarray(rows, np.int32), order.reshape(-1)])
-        dev = torch.from_numpy(host).to(device)
-        z = len(rows)
-        hit = cache[key] = TilePlan(req=dev[:n], q0=dev[n:2 * n], cut=dev[2 * n:3 * n], z0=dev[3 * n:4 * n],
-                                    rows=dev[4 * n:4 * n + z], cut_tokens=z, cuts=cuts if z else 1, order=dev[4 * n + z:],
-                                    rounds=order.shape[0], seats=seats)
-    return hit
+        arrays = {"req": np.asarray(t_req, np.int32), "q0": np.asarray(t_q0, np.int32), "cut": np.asarray(t_cut, np.int32),
+                  "z0": np.asarray(t_z0, np.int32), "rows": np.asarray(rows, np.int32), "order": order.reshape(-1),
+                  "singles": np.asarray(singles, np.int32)}
+        z, rounds = len(rows), order.shape[0]
+        longest_single = max((kv_lens[r] for r in singles), default=0)
+
+        def finish(views: Dict[str, torch.Tensor]) -> "TilePlan":
+            return TilePlan(req=views["req"], q0=views["q0"], cut=views["cut"], z0=views["z0"], rows=views["rows"],
+                            cut_tokens=z, cuts=cuts if z else 1, order=views["order"], rounds=rounds, seats=seats,
+                            singles=singles, single_ids=views["singles"], longest_single=longest_single)
+
+        return arrays, finish
+
+
+@functools.lru_cache(maxsize=None)
+def attention_planner(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int,
+                      device) -> Optional[AttentionPlanner]:
+    """The planner for a mixer of these sizes, or None when the general kernel serves it."""
+    if dtype != torch.bfloat16 or head_dim not in (64, 128) or page_size % 16:
+        return None
+    tile_rows = attention_tile_rows(num_heads, num_kv_heads, head_dim)
+    if tile_rows < 1:
+        return None
+    units = torch.cuda.get_device_properties(device).multi_processor_count
+    return AttentionPlanner(tile_rows, int(window), num_kv_heads, num_heads // num_kv_heads <= 16, units)
+
+
+def upload_arrays(arrays: Dict[str, np.ndarray], device) -> Dict[str, torch.Tensor]:
+    """Concatenate int32 arrays (each padded to 16 bytes), copy once, return device views."""
+    offsets, total = {}, 0
+    for name, arr in arrays.items():
+        offsets[name] = (total, arr.size)
+        total += (arr.size + 3) // 4 * 4
+    packed = np.zeros(max(total, 4), np.int32)
+    for name, arr in arrays.items():
+        o, n = offsets[name]
+        packed[o:o + n] = arr.reshape(-1)
+    dev = torch.from_numpy(packed).to(device)
+    return {name: dev[o:o + n] for name, (o, n) in offsets.items()}
+
+
+def _tile_plan(ctx, planner: AttentionPlanner, device) -> "TilePlan":
+    """The step's plan: the one the step function uploaded with its metadata, or - for a caller
+    that made its context by hand - one made and uploaded here."""
+    plans = getattr(ctx, "plans", None)
+    if plans is None:
+        plans = ctx.plans = {}
+    plan = plans.get(planner)
+    if plan is None:
+        arrays, finish = planner.plan(ctx.q_lens, ctx.kv_lens)
+        plan = plans[planner] = finish(upload_arrays(arrays, device))
+    return plan
 
 
 @dataclass
@@ -300,6 +327,9 @@ class TilePlan:
     order: torch.Tensor        # [rounds, seats]: which entry a block takes in which round (-1: none)
     rounds: int
     seats: int
+    singles: Tuple[int, ...] = ()             # requests that bring one token beside requests that bring more
+    single_ids: Optional[torch.Tensor] = None  # the same on the device
+    longest_single: int = 0                   # the longest context among them
 
 
 MAX_TILE_CUTS = 8
@@ -314,23 +344,6 @@ def cut_count(walks: List[int], seats_wanted: int) -> int:
         return 1
     cuts = min(MAX_TILE_CUTS, seats_wanted // tiles, max(walks) // 2)
     return max(1, cuts)
-
-
-def _single_tokens(ctx, device):
-    """The step's requests that bring exactly one token, beside requests that bring more: their
-    indices (host tuple and device int32), cached on the step."""
-    hit = getattr(ctx, "_single_tokens", None)
-    if hit is None:
-        singles = tuple(r for r, n in enumerate(ctx.q_lens) if n == 1)
-        if len(singles) == len(ctx.q_lens):
-            singles = ()
-        ids = torch.tensor(singles, dtype=torch.int32).to(device) if singles else None
-        hit = (singles, ids)
-        try:
-            ctx._single_tokens = hit
-        except AttributeError:
-            pass
-    return hit
 
 
 def decode_length_bucket(max_kv_len: int) -> int:
@@ -350,37 +363,47 @@ def decode_splits(R: int, num_kv_heads: int, max_kv_len: int) -> int:
     return min(splits, max(1, decode_length_bucket(max_kv_len) // DECODE_MIN_KEYS_PER_SPLIT))
 
 
+def _attn_part(ws: Optional[KernelWorkspace], floats: int, device) -> torch.Tensor:
+    return ws.attn_part if ws is not None else torch.empty(max(4, floats), dtype=torch.float32, device=device)
+
+
+def _decode_splits_that_fit(ws, n_req: int, num_heads: int, num_kv_heads: int, head_dim: int, longest: int) -> int:
+    splits = decode_splits(n_req, num_kv_heads, longest)
+    if ws is not None:
+        while splits > 1 and n_req * num_heads * splits * (head_dim + 4) > ws.attn_part.numel():
+            splits -= 1
+    return splits
+
+
 def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
-                    page_size, scale, window, pages) -> bool:
+                    page_size, scale, window, pages, ws: Optional[KernelWorkspace] = None) -> bool:
     if head_dim not in (64, 128) or page_size % 16 or q.data_ptr() % 16 or q.stride(0) % 8 or out.stride(0) % 4:
         return False
     G = num_heads // num_kv_heads
     R = ctx.R
+
     def decode_kernel(n_req: int, req_ids: int, longest: int) -> None:
-        splits = decode_splits(n_req, num_kv_heads, longest)
-        ws = workspace(q.device)
-        while splits > 1 and n_req * num_heads * splits * (head_dim + 4) > ws.attn_part.numel():
-            splits -= 1
+        splits = _decode_splits_that_fit(ws, n_req, num_heads, num_kv_heads, head_dim, longest)
+        part = _attn_part(ws, n_req * num_heads * splits * (head_dim + 4), q.device)
         _lib.call("bf16", "pi_attention_decode", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
                   k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
                   ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), req_ids, n_req, num_heads, num_kv_heads, head_dim,
-                  page_size, float(scale), int(window), pages, splits, ws.attn_part.data_ptr(), ws.attn_part.numel(),
-                  _stream())
+                  page_size, float(scale), int(window), pages, splits, part.data_ptr(), part.numel(), _stream())
 
     if ctx.all_decode and G <= 16:
         decode_kernel(R, 0, ctx.max_kv_len)
         return True
-    tile_rows = attention_tile_rows(num_heads, num_kv_heads, head_dim)
-    if tile_rows < 1:
+    planner = attention_planner(q.dtype, num_heads, num_kv_heads, head_dim, page_size, window, q.device)
+    if planner is None:
         return False
     # A step of prompt portions and single tokens: the single tokens, whose keys no other token
     # of the step shares, go to the key-split kernel (a tile of one token would walk its whole
     # context in one block, mostly on padding); the portions go to the tile kernel.
-    singles, single_ids = _single_tokens(ctx, q.device) if G <= 16 else ((), None)
-    if singles:
-        decode_kernel(len(singles), single_ids.data_ptr(), max(ctx.kv_lens[r] for r in singles))
-    plan = _tiles(ctx, tile_rows, int(window), num_kv_heads, q.device, skip=singles)
-    tile_part = workspace(q.device).tile_part_for(plan.cut_tokens * num_heads * plan.cuts * (head_dim + 4))
+    plan = _tile_plan(ctx, planner, q.device)
+    if plan.singles:
+        decode_kernel(len(plan.singles), plan.single_ids.data_ptr(), plan.longest_single)
+    floats = plan.cut_tokens * num_heads * plan.cuts * (head_dim + 4)
+    tile_part = ws.tile_part_for(floats) if ws is not None else torch.empty(max(4, floats), dtype=torch.float32, device=q.device)
     _lib.call("bf16", "pi_attention_prefill_mfma", out.data_ptr(), out.stride(0), q.data_ptr(), q.stride(0),
               k_cache.data_ptr(), v_cache.data_ptr(), block_table.data_ptr(), block_table.shape[1],
               ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), plan.req.data_ptr(), plan.q0.data_ptr(), plan.cut.data_ptr(),
@@ -393,7 +416,8 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
 
 
 def decode_attention_from_projection(out, qkv, ctx, table, num_heads, num_kv_heads, head_dim, k_cache, v_cache,
-                                     block_table, page_size, scale, window, pages, write_kv) -> bool:
+                                     block_table, page_size, scale, window, pages, write_kv,
+                                     ws: Optional[KernelWorkspace] = None) -> bool:
     """A step of single tokens: attention straight from the q|k|v projection (``qkv``: a bfloat16
     tensor [T, N] or ``Partials``), which the kernel rotates by ``table`` (the step's cos / sin
     table [T, head_dim], or None) and whose keys and values it stores.  False: not for these sizes."""
@@ -407,23 +431,13 @@ def decode_attention_from_projection(out, qkv, ctx, table, num_heads, num_kv_hea
         return False
     if (qkv.N % 4 or qkv.part.data_ptr() % 16) if pieces else (qkv.stride(0) % 8 or qkv.stride(1) != 1 or qkv.data_ptr() % 16):
         return False
-    splits = decode_splits(R, num_kv_heads, ctx.max_kv_len)
-    ws = workspace(out.device)
-    while splits > 1 and R * num_heads * splits * (head_dim + 4) > ws.attn_part.numel():
-        splits -= 1
+    splits = _decode_splits_that_fit(ws, R, num_heads, num_kv_heads, head_dim, ctx.max_kv_len)
+    part = _attn_part(ws, R * num_heads * splits * (head_dim + 4), out.device)
     _lib.call("bf16", "pi_attention_decode_fused", out.data_ptr(), out.stride(0),
               None if pieces else qkv.data_ptr(), 0 if pieces else qkv.stride(0),
               qkv.part.data_ptr() if pieces else None, qkv.splits if pieces else 0, qkv.N if pieces else 0, R,
               None if table is None else table.data_ptr(), int(bool(write_kv)), k_cache.data_ptr(), v_cache.data_ptr(),
               block_table.data_ptr(), block_table.shape[1], ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), R, num_heads,
-              num_kv_heads, head_dim, page_size, float(scale), int(window), pages, splits, ws.attn_part.data_ptr(),
-              ws.attn_part.numel(), _stream())
+              num_kv_heads, head_dim, page_size, float(scale), int(window), pages, splits, part.data_ptr(),
+              part.numel(), _stream())
     return True
-
-
-def plan_attention(q_lens, kv_lens) -> dict:
-    return {}
-
-
-def attach_attention_plan(ctx, plan, views) -> None:
-    pass

@@ -68,6 +68,16 @@ class PagedAttention(Mixer):
     def cache_spec(self):
         return KVCacheSpec(self.num_kv_heads, self.head_dim, self.window)
 
+    @property
+    def graph_safe(self) -> bool:
+        # the kernels take the step's shape from device memory; a position encoding applied by
+        # library calls must make the promise itself
+        return self.position is None or bool(self.position.graph_safe)
+
+    def step_planner(self, page_size: int):
+        return ops.attention_planner(self.dtype, self.num_heads, self.num_kv_heads, self.head_dim, page_size,
+                                     self.window or 0, self.device)
+
     def load(self, tensors: Dict[str, torch.Tensor], dtype, device) -> None:
         super().load(tensors, dtype, device)
         mats = [tensors["q_proj.weight"]]
@@ -87,14 +97,15 @@ class PagedAttention(Mixer):
         rotary = self.position.rotary_params(ctx) if self.position is not None else None
         fused_position = self.position is None or rotary is not None
         table = ctx.block_tables[cache.group]
-        qkv = ops.qkv_projection(h, self.w_qkv, self.dtype) if fused_position else None
+        ws = ctx.workspace
+        qkv = ops.qkv_projection(h, self.w_qkv, self.dtype, ws) if fused_position else None
         if qkv is not None and ctx.all_decode:
             # single tokens only: one kernel rotates, writes the cache and attends
             attn = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
             if ops.decode_attention_from_projection(attn, qkv, ctx, rotary, self.num_heads, self.num_kv_heads,
                                                     self.head_dim, cache.k, cache.v, table, cache.page_size, self.scale,
-                                                    self.window or 0, writes):
-                ops.gemm(x, attn, self.w_o, accumulate=True, may_defer=True)
+                                                    self.window or 0, writes, ws):
+                ops.gemm(x, attn, self.w_o, accumulate=True, may_defer=True, ws=ws)
                 return
         if qkv is not None and not isinstance(qkv, torch.Tensor):
             # the projection is still in pieces (split over k): the rotation kernel sums them
@@ -105,7 +116,7 @@ class PagedAttention(Mixer):
         else:
             if qkv is None:
                 qkv = torch.empty((T, self.w_qkv.shape[0]), dtype=self.dtype, device=h.device)
-                ops.gemm(qkv, h, self.w_qkv)
+                ops.gemm(qkv, h, self.w_qkv, ws=ws)
             q = qkv[:, : self.q_size]
             k = qkv[:, self.q_size : self.q_size + self.kv_size] if self.own_kv else None
             v = qkv[:, self.q_size + self.kv_size :] if self.own_kv else None
@@ -119,10 +130,10 @@ class PagedAttention(Mixer):
         ops.paged_attention(
             attn, q, cache.k, cache.v, table, ctx,
             self.num_heads, self.num_kv_heads, self.head_dim, cache.page_size,
-            self.scale, self.window or 0,
+            self.scale, self.window or 0, ws,
         )
         # the block's next norm reads x, so the product may stay in pieces until then
-        ops.gemm(x, attn, self.w_o, accumulate=True, may_defer=True)
+        ops.gemm(x, attn, self.w_o, accumulate=True, may_defer=True, ws=ws)
 
 
 MIXERS.register("attention", PagedAttention)

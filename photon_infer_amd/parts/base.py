@@ -73,16 +73,9 @@ class StepContext:
     max_q_len: int = 0
     max_kv_len: int = 0
     all_decode: bool = False
-    # attention work lists (device) made by the step function
-    decode_reqs: Optional[torch.Tensor] = None   # [Rd] requests with one token
-    num_decode: int = 0
-    tile_req: Optional[torch.Tensor] = None      # [NT] request of each query tile
-    tile_q0: Optional[torch.Tensor] = None       # [NT] first token (within the request's portion)
-    num_tiles: int = 0
-    tile_rows: int = 0
-    decode_splits: int = 1                       # key ranges per request in split-K decode
-    workspace: Any = None                        # engine-owned scratch tensors
-    host_slots: Sequence[int] = ()
+    host_slots: Sequence[int] = ()        # the requests' state slots, on the host
+    workspace: Any = None                 # the runner's ops.KernelWorkspace: scratch memory of the kernels
+    plans: Dict[Any, Any] = field(default_factory=dict)     # step planner -> what it made for this step
     scratch: Dict[Any, Any] = field(default_factory=dict)   # what parts share within one step; emptied per step
 
 
@@ -100,7 +93,17 @@ class LayerCache:
 
 # --------------------------------------------------------------------------- part bases
 class Part:
-    """Common behaviour: declare tensors, receive them, know the compute dtype."""
+    """Common behaviour: declare tensors, receive them, know the compute dtype.
+
+    ``graph_safe``: True promises that ``forward`` does the same launches, on the same addresses,
+    for every step of one batch size of single tokens - it reads nothing of the step on the host
+    (``ctx.host_slots``, ``ctx.q_lens``, ``ctx.kv_lens``, values of device tensors) and decides
+    nothing in Python from it.  Only then may a decode step be captured once as a HIP graph and
+    replayed; one part without the promise makes the whole model step eagerly.  The default is
+    False: a part has to say so.
+    """
+
+    graph_safe = False
 
     def tensor_specs(self) -> List[TensorSpec]:
         return []
@@ -112,9 +115,10 @@ class Part:
 
 
 class Norm(Part):
-    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, ctx: Optional[StepContext] = None, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         """``x`` float32 [N, D] -> normalised rows in the compute dtype ([M, D] when
-        ``rows`` (int32 [M]) selects rows of ``x``)."""
+        ``rows`` (int32 [M]) selects rows of ``x``).  ``ctx`` is the step's context (None
+        when the norm is used on its own)."""
         raise NotImplementedError
 
 
@@ -135,6 +139,15 @@ class PositionEncoding(Part):
 class Mixer(Part):
     def cache_spec(self):
         """KVCacheSpec, StateSpec or None."""
+        return None
+
+    def step_planner(self, page_size: int):
+        """Called once after ``load``.  A mixer whose kernels want host-made work lists per step
+        returns a hashable *planner* with ``plan(q_lens, kv_lens) -> None | (arrays, finish)``:
+        ``arrays`` are int32 numpy arrays by name, which the step function packs into its one
+        upload of metadata, and ``finish(views)`` turns their device views into whatever the
+        mixer reads back from ``ctx.plans[planner]``.  Planners that compare equal run once per
+        step, for all their mixers.  None: nothing to plan."""
         return None
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:

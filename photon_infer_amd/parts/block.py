@@ -31,16 +31,20 @@ class PreNormBlock(Block):
         for prefix, part in self._named:
             part.load({n[len(prefix):]: t for n, t in tensors.items() if n.startswith(prefix)}, dtype, device)
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe for _, part in self._named)
+
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
         # A mixer or feed-forward may leave its update of x in pieces for the next norm to add
         # (ops.gemm(..., may_defer=True)).  A norm that does not go through ops.rmsnorm gets
         # the finished stream; mixers and feed-forwards always do, since a norm runs before them.
         if not getattr(self.norm1, "consumes_deferred", False):
-            ops.materialize(x)
-        self.mixer.forward(self.norm1.forward(x), x, ctx, cache)
+            ops.materialize(x, ctx.workspace)
+        self.mixer.forward(self.norm1.forward(x, ctx), x, ctx, cache)
         if not getattr(self.norm2, "consumes_deferred", False):
-            ops.materialize(x)
-        self.ffn.forward(self.norm2.forward(x), x, ctx)
+            ops.materialize(x, ctx.workspace)
+        self.ffn.forward(self.norm2.forward(x, ctx), x, ctx)
 
 
 BLOCKS.register("prenorm", PreNormBlock)

@@ -17,6 +17,8 @@ from .base import Part
 
 
 class TokenEmbedding(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int):
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
@@ -37,6 +39,8 @@ class TokenEmbedding(Part):
 
 
 class LMHead(Part):
+    graph_safe = True
+
     def __init__(self, vocab_size: int, hidden_size: int, tied: bool):
         self.vocab_size = int(vocab_size)
         self.hidden_size = int(hidden_size)
@@ -50,8 +54,8 @@ class LMHead(Part):
         super().load(tensors, dtype, device)
         self.weight = tied_weight if self.tied else tensors["weight"]
 
-    def forward(self, h: torch.Tensor) -> torch.Tensor:
+    def forward(self, h: torch.Tensor, ctx=None) -> torch.Tensor:
         """activations [M, hidden] -> float32 logits [M, vocab]."""
         logits = torch.empty((h.shape[0], self.vocab_size), dtype=torch.float32, device=h.device)
-        ops.gemm(logits, h, self.weight)
+        ops.gemm(logits, h, self.weight, ws=ctx.workspace if ctx is not None else None)
         return logits

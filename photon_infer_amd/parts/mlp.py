@@ -20,6 +20,8 @@ INTERLEAVE = 16   # rows of a matrix-core tile
 
 
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, hidden_size: int, intermediate_size: int, activation: str = "silu"):
         if activation != "silu":
             raise UnsupportedModelError(f"gated feed-forward activation '{activation}' is not supported")
@@ -54,8 +56,9 @@ class SwiGLU(FeedForward):
 
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
         act = torch.empty((h.shape[0], self.intermediate_size), dtype=self.dtype, device=h.device)
-        ops.gemm_swiglu(act, h, self.w_gate_up, self.interleave)
-        ops.gemm(x, act, self.w_down, accumulate=True, may_defer=True)   # the next norm reads x
+        ws = ctx.workspace if ctx is not None else None
+        ops.gemm_swiglu(act, h, self.w_gate_up, self.interleave, ws=ws)
+        ops.gemm(x, act, self.w_down, accumulate=True, may_defer=True, ws=ws)   # the next norm reads x
 
 
 FEED_FORWARDS.register("swiglu", SwiGLU)

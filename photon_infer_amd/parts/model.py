@@ -135,14 +135,22 @@ class DecoderModel:
     def forward(self, ctx: StepContext, caches: Sequence[LayerCache]) -> Optional[torch.Tensor]:
         """Run the step's tokens through the run order; float32 logits [M, vocab] at
         ``ctx.logit_rows`` (None when no row is wanted)."""
-        ops.reset_deferred()               # nothing of an earlier (failed) step may linger
+        ws = ctx.workspace
+        ops.reset_deferred(ws)             # nothing of an earlier (failed) step may linger
         ctx.scratch.clear()
         x = self.embedding.forward(ctx.token_ids)
         for i, entry in enumerate(self.spec.run_order):
             self.blocks[entry.layer].forward(x, ctx, caches[i])
         if ctx.logit_rows.shape[0] == 0:
-            ops.discard_deferred(x)        # the stream is not read again
+            ops.discard_deferred(x, ws)    # the stream is not read again
             return None
         if not getattr(self.final_norm, "consumes_deferred", False):
-            ops.materialize(x)
-        return self.head.forward(self.final_norm.forward(x, rows=ctx.logit_rows))
+            ops.materialize(x, ws)
+        return self.head.forward(self.final_norm.forward(x, ctx, rows=ctx.logit_rows), ctx)
+
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a decode step of this model may be captured as a HIP graph: every part of the
+        run order, the embedding, the final norm and the head promise it."""
+        parts = [self.embedding, self.final_norm, self.head] + [self.blocks[e.layer] for e in self.spec.run_order]
+        return all(getattr(p, "graph_safe", False) for p in parts)

@@ -18,6 +18,7 @@ from .base import NORMS, Norm
 
 class RMSNorm(Norm):
     consumes_deferred = True   # reads the stream through ops.rmsnorm, which adds a pending update
+    graph_safe = True
 
     def __init__(self, dim: int, eps: float):
         self.dim = int(dim)
@@ -31,10 +32,10 @@ class RMSNorm(Norm):
         super().load(tensors, dtype, device)
         self.weight = tensors["weight"]
 
-    def forward(self, x: torch.Tensor, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+    def forward(self, x: torch.Tensor, ctx=None, rows: Optional[torch.Tensor] = None) -> torch.Tensor:
         m = x.shape[0] if rows is None else rows.shape[0]
         out = torch.empty((m, self.dim), dtype=self.dtype, device=x.device)
-        ops.rmsnorm(out, x, self.weight, self.eps, rows)
+        ops.rmsnorm(out, x, self.weight, self.eps, rows, ws=ctx.workspace if ctx is not None else None)
         return out
 
 

@@ -46,6 +46,8 @@ def rope_frequencies(rotary_dim: int, theta: float, scaling=None) -> torch.Tenso
 
 
 class RotaryEmbedding(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, head_dim: int, theta: float, scaling=None, interleaved: bool = False,
                  rotary_dim: Optional[int] = None):
         self.head_dim = int(head_dim)

@@ -46,8 +46,10 @@ class SamplingParams:
 
 
 class Sampler:
-    def __init__(self, device):
+    def __init__(self, device, workspace=None):
+        """``workspace``: the runner's ``ops.KernelWorkspace`` (scratch of the sampling kernels)."""
         self.device = torch.device(device)
+        self.workspace = workspace
 
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], uniforms: Sequence[float]) -> List[int]:
         """One token per row of float32 ``logits`` [M, V]."""
@@ -56,9 +58,9 @@ class Sampler:
         if any(t > 0 for t in temperatures):
             host = np.asarray([list(temperatures), list(uniforms)], np.float32)
             dev = torch.from_numpy(host).to(logits.device)
-            ops.sample(out, logits, dev[0], dev[1])
+            ops.sample(out, logits, dev[0], dev[1], ws=self.workspace)
         else:
-            ops.sample(out, logits)
+            ops.sample(out, logits, ws=self.workspace)
         return out.cpu().tolist()
 
     def greedy(self, logits: torch.Tensor) -> List[int]:

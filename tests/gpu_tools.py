@@ -61,7 +61,6 @@ class PagedKV:
 def attention_ctx(q_lens: Sequence[int], kv_lens: Sequence[int], dtype) -> SimpleNamespace:
     """The fields of a StepContext that the attention kernels read, made as the step function makes them."""
     from photon_infer_amd import ops
-    from photon_infer_amd.engine.step import _upload
 
     R = len(q_lens)
     q_start = np.zeros(R + 1, np.int32)
@@ -71,14 +70,12 @@ def attention_ctx(q_lens: Sequence[int], kv_lens: Sequence[int], dtype) -> Simpl
         "req_of_token": np.repeat(np.arange(R, dtype=np.int32), q_lens),
         "q_start": q_start, "kv_len": np.asarray(kv_lens, np.int32),
     }
-    plan = ops.plan_attention(list(q_lens), list(kv_lens), dtype)
-    parts.update(plan.get("arrays", {}))
-    views = _upload(parts, DEV)
-    ctx = SimpleNamespace(T=int(sum(q_lens)), R=R, dtype=dtype, q_lens=list(q_lens), kv_lens=list(kv_lens),
-                          max_q_len=max(q_lens), max_kv_len=max(kv_lens), all_decode=all(n == 1 for n in q_lens), scratch={},
-                          **{k: views[k] for k in ("positions", "req_of_token", "q_start", "kv_len")})
-    ops.attach_attention_plan(ctx, plan, views)
-    return ctx
+    views = ops.upload_arrays(parts, DEV)
+    # no runner here: no workspace (the ops take what they need per call) and no plans made
+    # beforehand (the attention op makes its work list itself)
+    return SimpleNamespace(T=int(sum(q_lens)), R=R, dtype=dtype, q_lens=list(q_lens), kv_lens=list(kv_lens),
+                           max_q_len=max(q_lens), max_kv_len=max(kv_lens), all_decode=all(n == 1 for n in q_lens), scratch={},
+                           workspace=None, plans={}, **{k: views[k] for k in ("positions", "req_of_token", "q_start", "kv_len")})
 
 
 def run_trace(runner, steps: List[dict], out_dir: str) -> Dict[tuple, torch.Tensor]:

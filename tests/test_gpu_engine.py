@@ -16,7 +16,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 @pytest.fixture(scope="module")
 def model_dirs(tmp_path_factory):
     root = tmp_path_factory.mktemp("models")
-    return {name: make_model_dir(root, name, seed=21) for name in ("A", "B")}
+    return {name: make_model_dir(root, name, seed=21) for name in ("A", "B", "F")}
 
 
 def engine(model_dir, name, **kw):
@@ -39,10 +39,18 @@ def test_greedy_generation_equals_the_plain_implementation(model_dirs):
     assert eng.runner.cache.num_live == 0 and eng.runner.cache.free_pages() == 128
 
 
-def test_greedy_generation_in_bfloat16_follows_the_plain_arg_max(model_dirs):
-    cfg, W = P.read_model_folder(model_dirs["B"])
-    prompts = [random_tokens(n, 384, 40 + n) for n in (1, 7, 33)]
-    outs = engine(model_dirs["B"], "B", dtype="bfloat16", chunk_size=16).generate(prompts, max_new_tokens=10, ignore_eos=True)
+@pytest.mark.parametrize("name", ["B", "F"])
+def test_greedy_generation_in_bfloat16_follows_the_plain_arg_max(model_dirs, name):
+    # F: the kernels chosen at real sizes (products split over k, the two-kernel sampler), through
+    # the default engine: graphs and a step ahead
+    cfg, W = P.read_model_folder(model_dirs[name])
+    prompts = [random_tokens(n, ALL[name][0]["vocab_size"], 40 + n) for n in (1, 7, 33)]
+    eng = engine(model_dirs[name], name, dtype="bfloat16", chunk_size=16)
+    outs = eng.generate(prompts, max_new_tokens=10, ignore_eos=True)
+    assert eng.runner.graph_safe and eng.runner._graphs
+    if name == "F":
+        counts = eng.runner.workspace.counts
+        assert counts["deferred"] > 0 and counts["qkv_pieces"] > 0 and counts["added_by_norm"] > 0, counts
     for p, out in zip(prompts, outs):
         seq = list(p)
         assert len(out) == 10
@@ -140,7 +148,7 @@ def test_command_line(model_dirs, tmp_path):
     assert "User: hi there" in proc.stdout and "Prompt tokens: 9" in proc.stdout and "Assistant:" in proc.stdout
 
 
-@pytest.mark.parametrize("dtype,name", [("float32", "A"), ("bfloat16", "D")])
+@pytest.mark.parametrize("dtype,name", [("float32", "A"), ("bfloat16", "D"), ("bfloat16", "F")])
 def test_graph_replayed_decode_equals_eager_steps(tmp_path, dtype, name):
     """Decode-only steps replay a captured graph (model + sampling kernel); every replay must
     give what the eager step gives, with eager work (new requests' prompts) between replays."""
@@ -166,7 +174,7 @@ def test_graph_replayed_decode_equals_eager_steps(tmp_path, dtype, name):
     assert [len(x) for x in graphed] == [14, 17, 20, 9]
 
 
-@pytest.mark.parametrize("dtype,name", [("float32", "A"), ("bfloat16", "D")])
+@pytest.mark.parametrize("dtype,name", [("float32", "A"), ("bfloat16", "D"), ("bfloat16", "F")])
 def test_a_step_ahead_gives_the_same_tokens(tmp_path, dtype, name):
     """Launching the next decode step before this one's tokens are on the host (they are fed
     back on the device) changes nothing: requests of different lengths ending at different
@@ -250,6 +258,92 @@ def test_decode_steps_queued_far_ahead_of_the_gpu(tmp_path):
         return [o.tolist() for o in outs]
 
     assert run(True) == run(False)
+
+
+@pytest.mark.parametrize("lookahead", [False, True])
+def test_abort_of_waiting_running_and_launched_requests(model_dirs, lookahead):
+    """A cancelled request gives its slot and pages back at once, wherever it is: still waiting,
+    in the middle of its prompt, decoding, or in a decode step that was launched and not read.
+    The others generate what they generate without it; no page or slot is lost."""
+    prompts = [random_tokens(n, 256, 160 + n) for n in (6, 30, 11, 4, 9)]
+    want = engine(model_dirs["A"], "A", max_batch=3).generate(prompts, max_new_tokens=16, ignore_eos=True)
+    eng = engine(model_dirs["A"], "A", max_batch=3, chunk_size=8, max_step_tokens=12, lookahead=lookahead)
+    ids = [eng.add_request(p, 16, ignore_eos=True) for p in prompts]
+    eng.step()                                               # 0 through, 1 mid-prompt, 3 and 4 waiting (three slots)
+    r1 = eng.get_request(ids[1])
+    assert 0 < r1.num_computed_tokens < 30 and eng.get_request(ids[4]).state.value == "waiting"
+    free = eng.runner.cache.free_pages()
+    assert eng.abort(ids[1]) and eng.abort(ids[4])           # mid-prompt, and waiting
+    assert eng.runner.cache.free_pages() > free and r1.finish_reason == "aborted" and r1.generated_tokens == []
+    eng.runner.cache.check_invariants()
+    for _ in range(8):
+        eng.step()
+    r0 = eng.get_request(ids[0])
+    assert not r0.is_finished() and r0.num_generated() > 2
+    if lookahead:
+        assert eng._in_flight is not None and r0 in eng._in_flight.reqs      # a step with it is on the GPU, unread
+    had, live = list(r0.generated_tokens), eng.runner.cache.num_live
+    assert eng.abort(ids[0])
+    assert eng.runner.cache.num_live == live - 1             # before the launched step is read
+    eng.runner.cache.check_invariants()
+    eng.run_until_complete()
+    assert r0.generated_tokens == had == want[0][:len(had)] and r0.finish_reason == "aborted"
+    assert eng.get_result(ids[2]) == want[2] and eng.get_result(ids[3]) == want[3]
+    assert not eng.abort(ids[2])                             # finished long ago
+    assert eng.runner.cache.num_live == 0 and eng.runner.cache.free_pages() == 128
+    eng.runner.cache.check_invariants()
+    assert eng.get_stats().num_aborted == 3
+
+
+def test_the_default_pool_fits_the_device_and_too_much_is_a_typed_error(tmp_path):
+    """Without a pool size the engine takes every slot at the model's full length if that fits,
+    else a share of the memory that is free after the weights, and lets no sequence grow beyond
+    it; a size that was asked for and does not fit is an error of the engine's own, before any
+    allocation."""
+    from photon_infer_amd import ContinuousBatchEngine, ErrorCode, OutOfMemoryError, write_random_model
+    from photon_infer_amd.config import LlamaConfig
+    huge = LlamaConfig.from_dict(dict(ALL["A"][0], max_position_embeddings=1 << 30))
+    d = write_random_model(huge, str(tmp_path / "huge"), seed=1, std=0.02)
+    free, _ = torch.cuda.mem_get_info()
+    eng = ContinuousBatchEngine(d, dtype="bfloat16", block_size=16, max_batch=8, memory_fraction=0.02)
+    page_bytes = 2 * 2 * (2 * 16 * 16) * 2                  # layers x (k, v) x kv heads x head size x page x bytes
+    pool = eng.runner.num_pages * page_bytes
+    assert 0.01 * free < pool <= 0.021 * free
+    assert eng.runner.max_model_len == eng.runner.num_pages * 16 < (1 << 30)
+    assert eng.generate([[1, 2, 3]], max_new_tokens=4, ignore_eos=True)[0].__len__() == 4
+    del eng
+    small = ContinuousBatchEngine(d, dtype="bfloat16", block_size=16, max_batch=2, max_model_len=256)
+    assert small.runner.num_pages == 2 * 256 // 16 and small.runner.max_model_len == 256     # fits: every slot at full length
+    with pytest.raises(OutOfMemoryError, match="num_blocks=") as err:
+        ContinuousBatchEngine(d, dtype="bfloat16", block_size=16, num_blocks=1 << 34)
+    assert err.value.code == ErrorCode.OUT_OF_MEMORY and "GiB" in str(err.value)
+    with pytest.raises(OutOfMemoryError, match="max_cache_tokens="):
+        ContinuousBatchEngine(d, dtype="bfloat16", block_size=16, max_cache_tokens=1 << 40)
+
+
+def test_two_engines_stepping_in_turns_do_not_disturb_each_other(model_dirs):
+    """Every runner owns its kernel scratch and its pending residual update: two engines in one
+    process, stepped alternately (as two threads would interleave), generate what each generates
+    alone.  Model F leaves a product in pieces at the end of nearly every kernel sequence."""
+    prompts_a = [random_tokens(n, 32768, 140 + n) for n in (5, 40, 17)]
+    prompts_b = [random_tokens(n, 32768, 150 + n) for n in (23, 3)]
+
+    def make():
+        return engine(model_dirs["F"], "F", dtype="bfloat16", chunk_size=16, max_step_tokens=24)
+
+    alone_a = make().generate(prompts_a, max_new_tokens=12, temperature=0.7, seed=5, ignore_eos=True)
+    alone_b = make().generate(prompts_b, max_new_tokens=15, temperature=0.7, seed=9, ignore_eos=True)
+    ea, eb = make(), make()
+    assert ea.runner.workspace is not eb.runner.workspace
+    ids_a = [ea.add_request(p, 12, temperature=0.7, seed=5 + i, ignore_eos=True) for i, p in enumerate(prompts_a)]
+    ids_b = [eb.add_request(p, 15, temperature=0.7, seed=9 + i, ignore_eos=True) for i, p in enumerate(prompts_b)]
+    while ea.has_work() or eb.has_work():
+        if ea.has_work():
+            ea.step()
+        if eb.has_work():
+            eb.step()
+    assert [ea.get_result(i) for i in ids_a] == alone_a
+    assert [eb.get_result(i) for i in ids_b] == alone_b
 
 
 def test_cpp_program_generates_what_the_python_entry_point_generates(model_dirs, tmp_path):

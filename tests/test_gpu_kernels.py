@@ -60,6 +60,76 @@ def test_rmsnorm(_ops, D, out_dtype, w_dtype):
     assert torch.equal(out2, out[[6, 0, 3]])
 
 
+@pytest.mark.parametrize("D", [24, 1001, 2048, 4100])
+@pytest.mark.parametrize("splits", [1, 3, 4, 9])
+@pytest.mark.parametrize("out_dtype", [F32, BF16])
+def test_rmsnorm_adds_the_pieces_of_a_pending_update_first(_ops, D, splits, out_dtype):
+    """A product into the stream that was split over k waits in the workspace; the norm adds its
+    pieces (in split order), writes the sum back into the stream and normalises it, in one pass:
+    all rows, or only the rows it is asked for.  D = 1001 takes the general kernel, the others
+    the kernel with 16-byte accesses (one, one and two groups per thread)."""
+    from photon_infer_amd.ops.workspace import Partials, PendingUpdate
+    M = 7
+    x0 = torch.randn(M, D, generator=gen(D)) * 2 + 0.25
+    pieces = torch.randn(splits, M, D, generator=gen(D + splits))
+    w = (torch.rand(D, generator=gen(1)) + 0.5).to(out_dtype)
+    total = x0.double() + pieces.double().sum(0)
+    want = P.rmsnorm(total, w.double(), 1e-5)
+    tol = 3e-6 if out_dtype == F32 else 2 ** -8
+    for rows in (None, [5, 0, 3]):
+        ws = _ops.KernelWorkspace(DEV)
+        x = x0.clone().to(DEV)
+        ws.pending = PendingUpdate(x, Partials(pieces.to(DEV), splits, M, D))
+        sel = list(range(M)) if rows is None else rows
+        out = torch.full((len(sel), D), float("nan"), dtype=out_dtype, device=DEV)
+        _ops.rmsnorm(out, x, w.to(DEV), 1e-5, None if rows is None else torch.tensor(rows, dtype=torch.int32, device=DEV), ws=ws)
+        assert ws.pending is None and ws.counts["added_by_norm"] == 1
+        close(out, want[sel], tol, f"norm of stream + pieces, D={D} splits={splits} rows={rows}")
+        close(x[sel], total[sel], 1e-6, "the stream holds the sum afterwards")
+        others = [m for m in range(M) if m not in sel]
+        assert torch.equal(x[others].cpu(), x0[others])            # rows not asked for are left alone
+        # a second norm of the same stream finds nothing pending and the same values
+        again = torch.empty_like(out)
+        _ops.rmsnorm(again, x, w.to(DEV), 1e-5, None if rows is None else torch.tensor(rows, dtype=torch.int32, device=DEV), ws=ws)
+        assert torch.equal(again, out)
+    # a pending update of another stream is not this norm's to add
+    ws = _ops.KernelWorkspace(DEV)
+    other = torch.zeros(M, D, device=DEV)
+    ws.pending = PendingUpdate(other, Partials(pieces.to(DEV), splits, M, D))
+    x = x0.clone().to(DEV)
+    out = torch.empty(M, D, dtype=out_dtype, device=DEV)
+    _ops.rmsnorm(out, x, w.to(DEV), 1e-5, ws=ws)
+    assert ws.pending is not None and torch.equal(x.cpu(), x0)
+    close(out, P.rmsnorm(x0.double(), w.double(), 1e-5), tol, "norm beside another stream's pending update")
+
+
+def test_a_second_split_product_applies_the_first_ones_pieces(_ops):
+    """The workspace holds one product's pieces: a product that needs it applies the pending
+    update of the other stream before it overwrites them."""
+    M, N, K = 4, 512, 2048
+    a = (torch.randn(M, K, generator=gen(1)) * 0.25).to(BF16).to(DEV)
+    w1 = (torch.randn(N, K, generator=gen(2)) * 0.25).to(BF16).to(DEV)
+    w2 = (torch.randn(N, K, generator=gen(3)) * 0.25).to(BF16).to(DEV)
+    ws = _ops.KernelWorkspace(DEV)
+    x, y = torch.ones(M, N, device=DEV), torch.full((M, N), 2.0, device=DEV)
+    _ops.gemm(x, a, w1, accumulate=True, may_defer=True, ws=ws)
+    assert ws.pending is not None and ws.pending.is_for(x) and ws.counts["split_products"] == 1
+    _ops.gemm(y, a, w2, accumulate=True, may_defer=True, ws=ws)
+    assert ws.pending.is_for(y) and ws.counts["flushed"] == 1
+    _ops.materialize(y, ws)
+    close(x, 1.0 + a.double().cpu() @ w1.double().cpu().t(), 2e-6, "first stream")
+    close(y, 2.0 + a.double().cpu() @ w2.double().cpu().t(), 2e-6, "second stream")
+    # two workspaces never see each other's pieces
+    ws1, ws2 = _ops.KernelWorkspace(DEV), _ops.KernelWorkspace(DEV)
+    x, y = torch.ones(M, N, device=DEV), torch.full((M, N), 2.0, device=DEV)
+    _ops.gemm(x, a, w1, accumulate=True, may_defer=True, ws=ws1)
+    _ops.gemm(y, a, w2, accumulate=True, may_defer=True, ws=ws2)
+    assert ws1.pending.is_for(x) and ws2.pending.is_for(y) and ws1.counts["flushed"] == 0
+    _ops.materialize(x, ws1), _ops.materialize(y, ws2)
+    close(x, 1.0 + a.double().cpu() @ w1.double().cpu().t(), 2e-6, "first workspace")
+    close(y, 2.0 + a.double().cpu() @ w2.double().cpu().t(), 2e-6, "second workspace")
+
+
 def test_rmsnorm_reference_vectors(_ops):
     # tests/ops/test_rmsnorm.cpp:102-181
     x = torch.tensor([[1.0, 2.0, 3.0, 4.0], [2.0, 4.0, 6.0, 8.0]], device=DEV)
@@ -158,10 +228,16 @@ def test_gemm_on_large_tiles_split_over_k(_ops):
     base = torch.randn(M, N, generator=gen(3))
     want = a.double() @ w.double().t() + base.double()
     x = base.clone().to(DEV)
-    _ops.reset_deferred()
-    _ops.gemm(x, a.to(DEV), w.to(DEV), accumulate=True, may_defer=True)
-    _ops.materialize(x)
+    ws = _ops.KernelWorkspace(DEV)
+    _ops.gemm(x, a.to(DEV), w.to(DEV), accumulate=True, may_defer=True, ws=ws)
+    assert ws.pending is not None and ws.pending.pieces.splits > 1 and torch.equal(x.cpu(), base)   # nothing added yet
+    _ops.materialize(x, ws)
+    assert ws.pending is None and ws.counts["applied"] == 1
     close(x, want, 2e-6, "k-split large gemm")
+    # without a workspace nothing is ever left pending: the same product is finished by the call
+    y = base.clone().to(DEV)
+    _ops.gemm(y, a.to(DEV), w.to(DEV), accumulate=True, may_defer=True)
+    close(y, want, 2e-6, "large gemm without a workspace")
 
 
 @pytest.mark.parametrize("M,I,K", [(1000, 6160, 200), (1000, 6160, 192), (2048, 8192, 64)])

@@ -65,9 +65,7 @@ def test_swiglu_part(dtype):
     h = torch.randn(T, D, generator=gen(5)).to(dtype)
     x0 = torch.randn(T, D, generator=gen(6))
     x = x0.clone().to(DEV)
-    ffn.forward(h.to(DEV), x, None)
-    from photon_infer_amd import ops
-    ops.materialize(x)          # the product may still be in pieces for a norm to add
+    ffn.forward(h.to(DEV), x, None)          # no step context: no workspace, nothing is left pending
     Wr = {k: v.to(dtype).float() for k, v in W.items()}
     rd = (lambda t: t) if dtype == F32 else P.bf16_round
     act = rd(P.swiglu(rd(P.linear(h.float(), Wr["gate_proj.weight"])), rd(P.linear(h.float(), Wr["up_proj.weight"]))))
@@ -100,7 +98,6 @@ def test_attention_part(dtype, window):
         ctx.block_tables = {0: table}
         xs = x[lo:hi]
         attn.forward(h[lo:hi].to(DEV), xs, ctx, cache)
-        ops.materialize(xs)
     Wr = {k: v.to(dtype).float() for k, v in W.items()}
     rd = (lambda t: t) if dtype == F32 else P.bf16_round
     f = P.rope_frequencies(hd, 10000.0, None)
@@ -275,6 +272,44 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
         got = torch.cat(out[r])
         assert got.shape == want[r].shape
         assert (got - want[r]).abs().max() < 3e-5 * want[r].abs().max().clamp(min=1), r
+
+
+def test_toy_mixer_with_state_generates_through_the_engine(tmp_path):
+    """The toy's mixer reads the requests' slots on the host, so it does not promise that its
+    launches repeat (``graph_safe`` stays False): the engine with its default options (graphs,
+    a step ahead) must notice and step it eagerly.  More requests than slots, so that slots and
+    their state rows are used again; some greedy, some sampled."""
+    from photon_infer_amd import ContinuousBatchEngine, write_random_model
+    from photon_infer_amd.sampling import uniform_draw
+    ToyConfig = register_toy()
+    cfg = ToyConfig("ToyForCausalLM", hidden_size=48, vocab_size=97, num_heads=3, eps=1e-5)
+    d = write_random_model(cfg, str(tmp_path / "toy"), seed=3, std=0.15, norm_init="uniform", dtype="float32")
+    raw, W = P.read_model_folder(d)
+    eng = ContinuousBatchEngine(d, dtype="float32", block_size=4, num_blocks=48, max_batch=2, chunk_size=5)
+    assert eng.options.use_graphs and eng.options.lookahead
+    assert not eng.runner.graph_safe
+    prompts = [random_tokens(n, 97, 10 + n) for n in (7, 3, 12, 5, 9)]
+    new = [6, 11, 4, 9, 7]
+    temps = [0.0, 0.8, 0.0, 0.0, 1.3]
+    ids = [eng.add_request(p, n, temperature=t, seed=100 + i, ignore_eos=True) for i, (p, n, t) in enumerate(zip(prompts, new, temps))]
+    eng.run_until_complete()
+    assert not eng.runner._graphs                      # nothing was captured
+    assert eng.runner.cache.num_live == 0
+    for i, rid in enumerate(ids):
+        got = eng.get_result(rid)
+        assert len(got) == new[i]
+        seq = list(prompts[i])
+        for k, tok in enumerate(got):
+            logits = plain_toy(raw, W, seq)[-1]
+            if temps[i] == 0.0:
+                assert logits[tok].item() >= logits.max().item() - 1e-4, (i, k)
+            else:
+                assert tok == P.sample_temperature(logits, temps[i], uniform_draw(100 + i, k)), (i, k)
+            seq.append(tok)
+    # the Llama parts all make the promise
+    from tiny_models import make_model_dir
+    llama = ContinuousBatchEngine(make_model_dir(tmp_path, "A"), dtype="float32", block_size=4, num_blocks=16, max_batch=2)
+    assert llama.runner.graph_safe
 
 
 # ------------------------------------------------------------------ a second toy: routing and another position scheme

@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DTYPES = ["float32", "bfloat16"]
-MODELS = ["A", "B", "C", "D", "E"]
+MODELS = ["A", "B", "C", "D", "E", "F"]
 
 _plain_cache = {}
 
@@ -62,7 +62,23 @@ def check(got, model_dir, reqs, dtype, what):
     return worst
 
 
-LENGTHS = {"A": [5, 9, 17, 70, 128], "B": [1, 7, 33, 64, 100, 200], "C": [3, 48, 131], "D": [1, 31, 65, 300], "E": [2, 33, 129, 260]}
+LENGTHS = {"A": [5, 9, 17, 70, 128], "B": [1, 7, 33, 64, 100, 200], "C": [3, 48, 131], "D": [1, 31, 65, 300], "E": [2, 33, 129, 260],
+           "F": [1, 140, 300]}
+
+
+def check_kernel_selection(runner, name, dtype, portions=True, single_tokens=True):
+    """Model F is there so that the kernels chosen at real sizes run inside these comparisons: in
+    bfloat16 its o and down projections are split over k and left in pieces that the next norm
+    adds, and its q|k|v projection reaches the rotation (portions) or the fused decode kernel
+    (single tokens) in pieces.  The workspace counts say whether a run went that way."""
+    counts = runner.workspace.counts
+    if name != "F" or dtype != "bfloat16":
+        if dtype == "float32":
+            assert not counts, counts                   # the general kernels split nothing
+        return
+    assert counts["split_products"] > 0 and counts["deferred"] > 0 and counts["qkv_pieces"] > 0, counts
+    assert counts["added_by_norm"] == counts["deferred"] - counts["flushed"] - counts["applied"] - counts["discarded"], counts
+    assert counts["flushed"] == 0, counts               # every pending update found its norm
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -75,30 +91,34 @@ def test_each_request_alone_and_whole(model_dirs, tmp_path, name, dtype):
     runner = runner_for(model_dirs[name], name, dtype, live_token_need(steps))
     got = run_trace(runner, steps, str(tmp_path))
     check(got, model_dirs[name], reqs, dtype, "whole")
+    check_kernel_selection(runner, name, dtype)
     assert runner.cache.num_live == 0 and runner.cache.free_pages() == runner.num_pages
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", MODELS)
 def test_last_32_tokens_one_by_one(model_dirs, tmp_path, name, dtype):
-    n = {"A": 100, "B": 180, "C": 150, "D": 260, "E": 200}[name]
+    n = {"A": 100, "B": 180, "C": 150, "D": 260, "E": 200, "F": 290}[name]
     reqs = requests_for(name, [n], seed=1)
     toks = reqs["r0"]
     steps = cut_steps("r0", toks, [n - 32] + [1] * 32)
     runner = runner_for(model_dirs[name], name, dtype, live_token_need(steps))
     check(run_trace(runner, steps, str(tmp_path)), model_dirs[name], reqs, dtype, "tail decoded")
+    check_kernel_selection(runner, name, dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", MODELS)
 def test_portions_of_changing_size(model_dirs, tmp_path, name, dtype):
-    n = {"A": 120, "B": 230, "C": 170, "D": 290, "E": 210}[name]
+    n = {"A": 120, "B": 230, "C": 170, "D": 290, "E": 210, "F": 280}[name]
     reqs = requests_for(name, [n], seed=2)
-    for sizes in ([7, 2, 16, 3, 2, 33, 1, 5], [2], [64, 2, 2, 19]):
+    # F also in portions that the tile kernels take (more than 128 tokens), split over k
+    for sizes in ([7, 2, 16, 3, 2, 33, 1, 5], [2], [64, 2, 2, 19]) + (([130, 2, 140],) if name == "F" else ()):
         steps = cut_steps("r0", reqs["r0"], sizes)
         runner = runner_for(model_dirs[name], name, dtype, live_token_need(steps))
         check(run_trace(runner, steps, str(tmp_path / f"s{sizes[0]}_{len(sizes)}")), model_dirs[name], reqs, dtype,
               f"portions {sizes}")
+        check_kernel_selection(runner, name, dtype)
 
 
 def mixed_trace(reqs, patterns, max_live=4):
@@ -137,7 +157,7 @@ def mixed_trace(reqs, patterns, max_live=4):
 def test_mixed_requests_with_pages_used_again(model_dirs, tmp_path, name, dtype):
     lengths = {"A": [40, 9, 128, 77, 5, 100, 64, 30], "B": [100, 1, 33, 250, 64, 7, 180, 90],
                "C": [131, 48, 3, 200, 96, 150], "D": [300, 65, 2, 129, 500, 17, 210],
-               "E": [260, 33, 2, 129, 400, 64, 97]}[name]
+               "E": [260, 33, 2, 129, 400, 64, 97], "F": [300, 65, 2, 129, 260, 17, 210]}[name]
     reqs = requests_for(name, lengths, seed=3)
     pats = [[16, 1, 1, 1, 2], [1], [33, 2, 7], [64, 1, 1], [5, 3, 2], [2, 2, 50], [1, 1, 1, 40], [9]]
     patterns = {rid: pats[i % len(pats)] for i, rid in enumerate(reqs)}
@@ -161,6 +181,7 @@ def test_mixed_requests_with_pages_used_again(model_dirs, tmp_path, name, dtype)
     got = run_trace(runner, steps, str(tmp_path))
     assert any(len(v) > 1 for v in owners.values()), "no page was handed out a second time"
     check(got, model_dirs[name], reqs, dtype, "mixed")
+    check_kernel_selection(runner, name, dtype)
     runner.cache.check_invariants()
     assert runner.cache.num_live == 0 and runner.cache.free_pages() == runner.num_pages
 

@@ -198,3 +198,49 @@ def test_random_workloads_keep_every_invariant(seed):
             assert r.num_generated() == r.max_new_tokens
     assert cache.num_live == 0 and cache.free_pages() == cache.groups[0].pool.num_pages
     cache.check_invariants()
+
+
+def test_abort_gives_slot_and_pages_back_at_once():
+    cache, s = make(pages=16, page=4, slots=2, budget=16, chunk=8)
+    a = s.add_request(list(range(10)), SamplingParams(max_new_tokens=50))
+    b = s.add_request(list(range(6)), SamplingParams(max_new_tokens=50))
+    c = s.add_request(list(range(5)), SamplingParams(max_new_tokens=4))      # waits: two slots only
+    for _ in range(3):
+        run_step(cache, s, s.schedule_next_batch())
+    ra, rb, rc = (s.get_request(i) for i in (a, b, c))
+    assert ra.state is RequestState.RUNNING and rb.state is RequestState.RUNNING and rc.state is RequestState.WAITING
+    held = cache.free_pages()
+    assert s.abort(c)                                        # waiting: leaves the queue, holds nothing
+    assert rc.is_finished() and rc.finish_reason == "aborted" and not s.waiting and cache.free_pages() == held
+    generated = list(ra.generated_tokens)
+    assert s.abort(a)                                        # running: pages and slot are back before the next step
+    assert ra.finish_reason == "aborted" and ra.generated_tokens == generated
+    assert cache.free_pages() > held and cache.free_slots == 1 and ra not in s.running
+    cache.check_invariants()
+    assert not s.abort(a) and not s.abort(12345)             # finished, unknown
+    d = s.add_request(list(range(7)), SamplingParams(max_new_tokens=3))
+    while s.has_work():                                      # the freed slot serves the next request
+        run_step(cache, s, s.schedule_next_batch())
+    assert s.get_request(d).finish_reason == "length" and rb.finish_reason == "length"
+    assert cache.free_pages() == 16 and cache.num_live == 0
+    st = s.get_stats()
+    assert st.num_aborted == 2 and st.num_finished == 4
+
+
+@pytest.mark.parametrize("seed", range(5))
+def test_random_aborts_lose_no_page(seed):
+    rng = random.Random(seed)
+    cache, s = make(pages=24, page=4, slots=3, budget=12, chunk=5, max_len=64)
+    ids = []
+    for step in range(200):
+        if rng.random() < 0.3 and len(ids) < 25:
+            ids.append(s.add_request([1] * rng.randint(1, 30), SamplingParams(max_new_tokens=rng.randint(1, 12))))
+        if ids and rng.random() < 0.15:
+            s.abort(rng.choice(ids))
+        if s.has_work():
+            run_step(cache, s, s.schedule_next_batch())
+    for i in ids:
+        s.abort(i)
+    cache.check_invariants()
+    assert cache.free_pages() == 24 and cache.num_live == 0 and not s.has_work()
+    assert all(s.get_request(i).is_finished() for i in ids)

@@ -4,7 +4,8 @@ import random
 import numpy as np
 import pytest
 
-from photon_infer_amd.ops.fast import MAX_TILE_CUTS, cut_count, deal_tiles, decode_length_bucket, decode_splits
+from photon_infer_amd.ops.fast import (MAX_TILE_CUTS, AttentionPlanner, cut_count, deal_tiles, decode_length_bucket,
+                                        decode_splits)
 
 
 @pytest.mark.parametrize("seed", range(5))
@@ -50,3 +51,48 @@ def test_key_ranges_of_tiles_are_cut_only_when_the_tiles_are_few():
     assert cut_count([64] * 2, 64) == MAX_TILE_CUTS
     assert cut_count([5] * 16, 64) == 2                                         # a share keeps two rounds at least
     assert cut_count([1] * 4, 64) == 1
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_a_step_plan_covers_every_token_of_every_portion_once(seed):
+    """The planner of the prompt-attention kernel, on the host: tiles (or the shares of a cut tile)
+    cover each token of each portion exactly once; requests with one token go to the other kernel
+    when the planner says so; every entry is dealt to a block exactly once."""
+    rng = random.Random(seed)
+    R = rng.randint(1, 6)
+    q_lens = [rng.choice([1, 1, 2, 17, 64, 65, 300]) for _ in range(R)]
+    if all(n == 1 for n in q_lens):
+        q_lens[0] = 40
+    kv_lens = [n + rng.choice([0, 5, 700, 3000]) for n in q_lens]
+    apart = seed % 2 == 0
+    planner = AttentionPlanner(tile_rows=rng.choice([16, 32, 64]), window=rng.choice([0, 0, 100]), num_kv_heads=2,
+                               singles_apart=apart, units=rng.choice([8, 256]))
+    arrays, finish = planner.plan(q_lens, kv_lens)
+    assert all(a.dtype == np.int32 for a in arrays.values())
+    singles = [r for r, n in enumerate(q_lens) if n == 1] if apart else []
+    assert arrays["singles"].tolist() == singles
+    n = len(arrays["req"])
+    assert len(arrays["q0"]) == len(arrays["cut"]) == len(arrays["z0"]) == n
+    covered = {}
+    for r, q0, cut in zip(arrays["req"].tolist(), arrays["q0"].tolist(), arrays["cut"].tolist()):
+        share, shares = cut & 0xff, cut >> 8
+        assert 0 <= share < shares and r not in singles
+        covered.setdefault((r, q0), []).append((share, shares))
+    for (r, q0), shares in covered.items():
+        assert q0 % planner.tile_rows == 0 and q0 < q_lens[r]
+        assert sorted(s for s, _ in shares) == list(range(shares[0][1]))          # every share of a cut tile, once
+    for r, qn in enumerate(q_lens):
+        if r not in singles:
+            assert sorted(q0 for (rr, q0) in covered if rr == r) == list(range(0, qn, planner.tile_rows))
+    dealt = sorted(t for t in arrays["order"].tolist() if t >= 0)
+    assert dealt == list(range(n))
+    # rows of the cut tiles: one entry per token of every cut tile
+    cut_rows = sum(min(planner.tile_rows, q_lens[r] - q0) for (r, q0), sh in covered.items() if sh[0][1] > 1)
+    assert len(arrays["rows"]) == cut_rows
+
+
+def test_steps_of_single_tokens_need_no_plan_unless_the_tile_kernel_serves_them():
+    assert AttentionPlanner(16, 0, 2, True, 256).plan([1, 1, 1], [5, 900, 17]) is None
+    arrays, _ = AttentionPlanner(16, 0, 2, False, 256).plan([1, 1, 1], [5, 900, 17])
+    assert arrays["req"].tolist()[:3] == [0, 1, 2] or sorted(set(arrays["req"].tolist())) == [0, 1, 2]
+    assert arrays["singles"].size == 0

@@ -57,8 +57,23 @@ TINY_E = dict(
 )
 TINY_E_INIT = dict(std=0.06, norm_init="uniform", block_size=32)
 
+# Large enough that the kernels chosen at real sizes run inside the model: products whose k-range
+# is split (o, down and q|k|v: hidden >= 1024 and intermediate >= 2816 give K // 256 >= 2 and
+# K // 512 >= 2), their pieces added by the next norm, by the rotation and by the fused decode
+# kernel; four heads per kv head at head size 64; a vocabulary the two-kernel sampler takes; the
+# frequency scaling constants of the 1B model
+TINY_F = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=1024, intermediate_size=2816, num_hidden_layers=2,
+    num_attention_heads=16, num_key_value_heads=4, head_dim=64, vocab_size=32768, max_position_embeddings=1024,
+    rms_norm_eps=1e-5, rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    tie_word_embeddings=True,
+)
+TINY_F_INIT = dict(std=0.03, norm_init="uniform", block_size=16)
+
 ALL = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT), "D": (TINY_D, TINY_D_INIT),
-       "E": (TINY_E, TINY_E_INIT)}
+       "E": (TINY_E, TINY_E_INIT), "F": (TINY_F, TINY_F_INIT)}
 
 
 def make_model_dir(tmp_path, name: str, seed: int = 0, storage: str = "bfloat16") -> str:
