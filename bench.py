@@ -1,9 +1,9 @@
 #!/usr/bin/python3
-"""Decode and prefill throughput of the engine on one MI355X (Llama 3.2 1B layer sizes).
+"""Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode1b|serve3b|mixed8b]
 
-Prints ONE JSON line.  ``value`` is decoded tokens per second at batch 8 with the context
+Every workload prints ONE JSON line.  The default, ``decode1b`` (Llama 3.2 1B layer sizes):  ``value`` is decoded tokens per second at batch 8 with the context
 length of the benchmark configuration (every request's cache holds that many tokens when
 the timed steps end).  A "step" is one decode step of the whole batch through the engine's
 own path, driven as the engine drives its decode phase: metadata upload, the replayed graph
@@ -11,6 +11,18 @@ own path, driven as the engine drives its decode phase: metadata upload, the rep
 the copy of the chosen tokens to the host, which reads every step's tokens one step late.
 Also on the line: ``prefill`` (one 2,048-token prompt in one step), ``roofline`` (bytes the
 decode step has to read / its time, against 8 TB/s) and ``points`` (batch 1 and 64).
+``points`` also holds ``engine_b8``: decoded tokens per second of the same batch through
+``ContinuousBatchEngine`` (scheduler, request objects, sampling, the step ahead), measured over its
+decode phase.
+
+``--workload serve3b`` (Llama 3.2 3B layer sizes): continuous batching of 64 requests, prompts of
+128 to 2,048 tokens, 64 to 512 new tokens each, 16 there at the start and 4 more every 8 steps,
+through ``ContinuousBatchEngine``: total tokens per second, preemptions, share of the time the host
+waited for the GPU.  After demo/compare_batching_methods.cpp:251-309 of the reference.
+``--workload mixed8b`` (Llama 3.1 8B layer sizes): steps that hold one 512-token portion of a
+prompt late in a context of 8,192 beside 64 decoding requests at that context: milliseconds per
+mixed step, and the step's flops and bytes against the peaks.
+
 Weights are random (N(0, 0.02), norms 1), token ids uniform random; no dataset is involved.
 """
 from __future__ import annotations
@@ -33,6 +45,12 @@ MODEL = dict(
                       original_max_position_embeddings=8192),
     tie_word_embeddings=True, torch_dtype="bfloat16",
 )
+# the other two benchmark configurations
+MODEL_3B = dict(MODEL, hidden_size=3072, num_hidden_layers=28, num_attention_heads=24, num_key_value_heads=8, head_dim=128,
+                intermediate_size=8192)
+MODEL_8B = dict(MODEL, hidden_size=4096, num_hidden_layers=32, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+                intermediate_size=14336, tie_word_embeddings=False,
+                rope_scaling=dict(MODEL["rope_scaling"], factor=8.0))
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
 BLOCK_SIZE = 16
@@ -40,7 +58,7 @@ HBM_PEAK_GBS = 8000.0
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
 
 
-def make_runner(cfg_raw, layers, dtype, max_batch, max_cache_tokens, seed=0):
+def make_runner(cfg_raw, layers, dtype, max_batch, max_cache_tokens, seed=0, max_model_len=CONTEXT + 64, **options):
     import torch
 
     from photon_infer_amd.engine import EngineOptions, ModelRunner
@@ -58,7 +76,7 @@ def make_runner(cfg_raw, layers, dtype, max_batch, max_cache_tokens, seed=0):
         else:
             tensors[s.name] = (torch.randn(s.shape, generator=gen, device="cuda", dtype=torch.float32) * 0.02).to(tdtype)
     opts = EngineOptions(dtype="bfloat16" if dtype == "bf16" else "float32", block_size=BLOCK_SIZE,
-                         max_cache_tokens=max_cache_tokens, max_batch=max_batch, max_model_len=CONTEXT + 64)
+                         max_cache_tokens=max_cache_tokens, max_batch=max_batch, max_model_len=max_model_len, **options)
     return ModelRunner(None, opts, config=cfg, tensors=tensors), cfg
 
 
@@ -172,13 +190,178 @@ def time_prefill(runner, tokens, reps, seed=2):
     return (time.perf_counter() - t0) / reps
 
 
+def time_engine_decode(runner, batch, steps, warmup, context, seed=3):
+    """Seconds per decode step of ``batch`` requests through ContinuousBatchEngine with its default
+    options: the prompts run first (untimed, with ``warmup`` decode steps), then ``steps`` engine
+    steps are timed while every request decodes."""
+    import torch
+
+    from photon_infer_amd import ContinuousBatchEngine
+
+    eng = ContinuousBatchEngine(None, runner=runner)
+    g = torch.Generator().manual_seed(seed)
+    prompt_len = context - steps - warmup - 2
+    for _ in range(batch):
+        eng.add_request(torch.randint(0, runner.spec.vocab_size, (prompt_len,), generator=g).tolist(),
+                        steps + warmup + 2, ignore_eos=True)
+    reqs = list(eng.scheduler.requests.values())
+    while min(r.num_generated() for r in reqs) < warmup:
+        eng.step()
+    torch.cuda.synchronize()
+    n0, t0 = eng.steps, time.perf_counter()
+    while eng.steps - n0 < steps and eng.has_work():
+        eng.step()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / max(1, eng.steps - n0)
+    eng.run_until_complete()
+    return sec
+
+
+def workload_serve3b(args) -> int:
+    """Continuous batching at Llama 3.2 3B layer sizes (see the module text)."""
+    import collections
+    import random
+
+    import torch
+
+    from photon_infer_amd import ContinuousBatchEngine
+
+    layers = args.layers or MODEL_3B["num_hidden_layers"]
+    n_req, first, more, every = 64, 16, 4, 8
+    rng = random.Random(0)
+    shapes = [(rng.randint(128, 2048), rng.randint(64, 512)) for _ in range(n_req)]
+    cache_tokens = n_req * 2624            # every request at its longest, to the page
+    runner, cfg = make_runner(MODEL_3B, layers, args.dtype, n_req, cache_tokens, max_model_len=2048 + 512 + 64,
+                              max_step_tokens=2048, chunk_size=512)
+
+    def run():
+        eng = ContinuousBatchEngine(None, runner=runner)
+        g = torch.Generator().manual_seed(0)
+        pending = collections.deque(shapes)
+
+        def admit(n):
+            for _ in range(min(n, len(pending))):
+                p, o = pending.popleft()
+                eng.add_request(torch.randint(0, cfg.vocab_size, (p,), generator=g).tolist(), o, ignore_eos=True)
+
+        admit(first)
+        torch.cuda.synchronize()
+        t0, calls = time.perf_counter(), 0
+        while eng.has_work() or pending:
+            eng.step()
+            calls += 1
+            if calls % every == 0:
+                admit(more)
+        torch.cuda.synchronize()
+        return time.perf_counter() - t0, eng
+
+    run()                                   # untimed: captures the decode graphs of every batch size it meets
+    sec, eng = run()
+    reqs = list(eng.scheduler.requests.values())
+    generated = sum(r.num_generated() for r in reqs)
+    prompt = sum(p for p, _ in shapes)
+    assert generated == sum(o for _, o in shapes) and all(r.finish_reason == "length" for r in reqs)
+    stats = eng.get_stats()
+    elem = 2 if args.dtype == "bf16" else 4
+    line = {
+        "metric": "total tok/s (prompt + generated), continuous batching of 64 requests (Llama 3.2 3B layer sizes, random weights)",
+        "value": round((prompt + generated) / sec, 1), "unit": "tokens/s", "n_gpus": 1, "steps": eng.steps, "warmup": 0,
+        "ms_per_step": round(sec / eng.steps * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+        "config": {
+            "model": "llama-3.2-3b-sizes", "layers": layers, "layers_of_model": MODEL_3B["num_hidden_layers"],
+            "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+            "tied_embeddings": cfg.tie_word_embeddings, "requests": n_req, "prompt_lengths": "uniform 128..2048",
+            "output_lengths": "uniform 64..512", "admission": f"{first} at the start, {more} every {every} steps",
+            "chunk_size": 512, "max_step_tokens": 2048, "kv_block": BLOCK_SIZE, "cache_tokens": cache_tokens,
+            "parallelism": "single-gpu",
+        },
+        "seconds": round(sec, 3), "prompt_tokens": prompt, "generated_tokens": generated,
+        "generated_tok_per_s": round(generated / sec, 1), "preemptions": stats.num_preemptions,
+        "host_wait_share": round(eng.host_wait_seconds / sec, 3), "graphs": len(runner._graphs),
+        "weight_bytes": weight_bytes(runner), "kv_bytes_per_token": kv_bytes_per_token(cfg, layers, elem),
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+def workload_mixed8b(args) -> int:
+    """Mixed steps at Llama 3.1 8B layer sizes (see the module text)."""
+    import torch
+
+    from photon_infer_amd.engine import StepEntry
+
+    layers = args.layers or MODEL_8B["num_hidden_layers"]
+    ctx, portion, ndec = 8192, 512, 64
+    reps = max(2, min(4, args.steps))        # the timed portions cover the last 2,048 tokens of the context
+    runner, cfg = make_runner(MODEL_8B, layers, args.dtype, ndec + 1, (ndec + 1) * (ctx + 64), max_model_len=ctx + 64)
+    elem = 2 if args.dtype == "bf16" else 4
+    first = ctx - portion * (reps + 1)       # the portions that are timed end at ctx
+    rids = [f"d{i}" for i in range(ndec)]
+    for rid in rids:                         # the decoding requests: pages reserved, contents random
+        runner.admit(rid)
+        runner.cache.reserve(rid, ctx - reps - 2)
+        runner.cache.commit(rid, ctx - reps - 2)
+    runner.admit("p")
+    runner.cache.reserve("p", first)
+    runner.cache.commit("p", first)
+    for lc in runner.layer_caches:
+        lc.k.normal_()
+        lc.v.normal_()
+    g = torch.Generator().manual_seed(0)
+    prompt = torch.randint(0, cfg.vocab_size, (ctx,), generator=g).tolist()
+    state = {"pos": first}
+
+    def mixed():
+        p = state["pos"]
+        runner.step([StepEntry("p", prompt[p:p + portion], [])] + [StepEntry(r, [5], [0]) for r in rids])
+        state["pos"] = p + portion
+
+    mixed()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        mixed()
+    torch.cuda.synchronize()
+    sec = (time.perf_counter() - t0) / reps
+    tokens = portion + ndec
+    mean_ctx = ctx - portion * (reps - 1) / 2.0 - portion / 2.0       # keys a portion's token sees, averaged over the timed steps
+    per_layer = cfg.hidden_size * (cfg.q_size + 2 * cfg.kv_size) + cfg.q_size * cfg.hidden_size + 3 * cfg.hidden_size * cfg.intermediate_size
+    flops = 2.0 * tokens * per_layer * layers + 2.0 * ndec * cfg.hidden_size * cfg.vocab_size \
+        + layers * 4.0 * cfg.num_attention_heads * cfg.head_dim * (portion * mean_ctx + ndec * ctx)
+    kvb = kv_bytes_per_token(cfg, layers, elem)
+    step_bytes = weight_bytes(runner) + (ndec * ctx + mean_ctx + portion / 2.0) * kvb
+    line = {
+        "metric": "ms per mixed step: one 512-token prompt portion late in a context of 8192 beside 64 decoding requests (Llama 3.1 8B layer sizes, random weights)",
+        "value": round(sec * 1e3, 3), "unit": "ms", "n_gpus": 1, "steps": reps, "warmup": 1, "ms_per_step": round(sec * 1e3, 3),
+        "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": args.dtype,
+        "data": "synthetic: random weights N(0, 0.02), random cache contents, uniform random token ids",
+        "config": {
+            "model": "llama-3.1-8b-sizes", "layers": layers, "layers_of_model": MODEL_8B["num_hidden_layers"],
+            "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+            "tied_embeddings": cfg.tie_word_embeddings, "context": ctx, "portion_tokens": portion, "decoding_requests": ndec,
+            "kv_block": BLOCK_SIZE, "parallelism": "single-gpu",
+        },
+        "tokens_per_s": round(tokens / sec, 1),
+        "compute": {"flops": flops, "achieved": round(flops / sec / 1e12, 1), "peak": PEAK_FLOPS[args.dtype] / 1e12, "unit": "TFLOP/s",
+                    "frac": round(flops / sec / PEAK_FLOPS[args.dtype], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(step_bytes / sec / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(step_bytes / sec / 1e9 / HBM_PEAK_GBS, 4)},
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
     ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"],
+    ap.add_argument("--workload", choices=["decode1b", "serve3b", "mixed8b"], default="decode1b")
+    ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the model has, if memory or time needs it (both numbers are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 / 64 and prefill measurements")
@@ -194,6 +377,11 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU available", file=sys.stderr)
         return 1
+    if args.workload == "serve3b":
+        return workload_serve3b(args)
+    if args.workload == "mixed8b":
+        return workload_mixed8b(args)
+    args.layers = args.layers or MODEL["num_hidden_layers"]
     elem = 2 if args.dtype == "bf16" else 4
     big = 1 if (args.no_points or args.only) else 64
     runner, cfg = make_runner(MODEL, args.layers, args.dtype, max(big, args.batch), (max(big, args.batch)) * (CONTEXT + 64))
@@ -238,6 +426,7 @@ def main() -> int:
         for b in (1, 64):
             s, _ = time_decode(runner, b, args.steps, args.warmup, CONTEXT)
             points[f"decode_b{b}"] = round(b / s, 1)
+        points["engine_b8"] = round(args.batch / time_engine_decode(runner, args.batch, args.steps, args.warmup, CONTEXT), 1)
         line["points"] = points
     print(json.dumps(line), flush=True)
     return 0

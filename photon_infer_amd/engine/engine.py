@@ -8,6 +8,7 @@ are given as token ids (text goes through the tokenizer of the command line).
 from __future__ import annotations
 
 import sys
+import time
 from typing import Dict, List, Optional, Sequence
 
 from ..errors import RequestError
@@ -49,6 +50,7 @@ class ContinuousBatchEngine:
         self.sampler = Sampler(self.runner.device, self.runner.workspace)
         self.eos_token_ids = tuple(self.runner.spec.eos_token_ids)
         self.steps = 0
+        self.host_wait_seconds = 0.0     # time the host spent waiting for the GPU's tokens
         # a decode step that was launched and whose tokens have not been read yet
         self._in_flight: Optional[_InFlight] = None
         # pinned buffers the sampled tokens are copied to, by (batch size, turn)
@@ -139,7 +141,9 @@ class ContinuousBatchEngine:
 
     def _collect(self, fl: "_InFlight", skip: Sequence[InferenceRequest] = ()) -> List[InferenceRequest]:
         """Read a launched step's tokens and book them; returns the requests they finished."""
+        t0 = time.perf_counter()
         fl.done.synchronize()
+        self.host_wait_seconds += time.perf_counter() - t0
         done = []
         for req, tok in zip(fl.reqs, fl.host.tolist()):
             if req in skip:            # ended a step earlier; this token was computed for nothing
@@ -192,11 +196,16 @@ class ContinuousBatchEngine:
             if self.options.lookahead:
                 self._launch_decode(sampled_reqs)
                 return []                   # its tokens are read in the next call
-            tokens = self.runner.decode_step(entries, temps, draws).tolist()
+            ids = self.runner.decode_step(entries, temps, draws)
+            t0 = time.perf_counter()
+            tokens = ids.tolist()
+            self.host_wait_seconds += time.perf_counter() - t0
         else:
             logits = self.runner.step(entries)
             if sampled_reqs:
+                t0 = time.perf_counter()
                 tokens = self.sampler.sample(logits, temps, draws)
+                self.host_wait_seconds += time.perf_counter() - t0
         done = []
         for req, n in batch.items:
             req.add_computed_tokens(n)
