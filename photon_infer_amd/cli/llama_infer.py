@@ -92,11 +92,22 @@ def _prompts(args, tok: Optional[TikTokenizer]) -> List[tuple]:
     return out
 
 
+def _device_name(args) -> str:
+    """What the GPU calls itself (the reference prints its device the same way, demo/llama_infer.cpp)."""
+    try:
+        import torch
+        if torch.cuda.is_available():
+            return f"{torch.cuda.get_device_name(0)} (HIP)"
+    except Exception:          # the banner must not be what stops the program
+        pass
+    return "no GPU found"
+
+
 def main(argv=None) -> int:
     args = build_parser().parse_args(argv)
     print("PhotonInfer - LLaMA Inference Demo")
     print("===================================")
-    print("Device: MI355X (HIP)")
+    print(f"Device: {_device_name(args)}")
     print(f"Compute dtype: {args.dtype}\n")
     try:
         tok = None

@@ -38,6 +38,29 @@ HOST_MODULES = {"runtime", "api"}
 HOST_HEADERS = {"api": ["api/photon_engine.h"]}
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]
 
+
+def sanitize_flags() -> List[str]:
+    """Compiler and linker flags for the host modules from ``PHOTON_SANITIZE`` (for instance
+    ``address,undefined``): the libraries are then built beside the ordinary ones, as
+    ``libphoton_<module>.<sanitizers>.so``.  A program that loads an address-sanitized library
+    must itself start under that sanitizer's runtime; ``build_host_program`` builds such programs
+    whole.  Device code is never built with sanitizers."""
+    names = os.environ.get("PHOTON_SANITIZE", "").strip()
+    if not names:
+        return []
+    return [f"-fsanitize={names}", "-fno-omit-frame-pointer", "-fno-sanitize-recover=all", "-g", "-O1"]
+
+
+def build_host_program(sources: List[str], out_path: str, sanitize: str = "", extra_flags: List[str] = ()) -> str:
+    """Compile host-only C++ sources (absolute paths, or names under csrc/) into the program
+    ``out_path``, optionally under sanitizers (``sanitize="address,undefined"``)."""
+    flags = [f for f in HOST_FLAGS if f != "-fPIC"]
+    if sanitize:
+        flags += [f"-fsanitize={sanitize}", "-fno-omit-frame-pointer", "-fno-sanitize-recover=all", "-g", "-O1"]
+    paths = [s if os.path.isabs(s) else os.path.join(CSRC_DIR, s) for s in sources]
+    _run([_host_compiler(), *flags, *extra_flags, "-I", CSRC_DIR, *paths, "-o", out_path], os.path.basename(out_path))
+    return out_path
+
 ARCH = "gfx950"
 HIPCC_FLAGS = [
     f"--offload-arch={ARCH}", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
@@ -100,7 +123,7 @@ def _build_dir() -> str:
 
 def source_hash(module: str) -> str:
     host = module in HOST_MODULES
-    h = hashlib.sha256(" ".join(HOST_FLAGS if host else HIPCC_FLAGS).encode())
+    h = hashlib.sha256(" ".join(HOST_FLAGS + sanitize_flags() if host else HIPCC_FLAGS).encode())
     for name in MODULES[module] + (HOST_HEADERS.get(module, []) if host else HEADERS):
         h.update(" ".join(FILE_FLAGS.get(name, [])).encode())
         path = os.path.join(CSRC_DIR, name)
@@ -111,7 +134,8 @@ def source_hash(module: str) -> str:
 
 
 def library_path(module: str) -> str:
-    return os.path.join(_build_dir(), f"libphoton_{module}.so")
+    tag = os.environ.get("PHOTON_SANITIZE", "").strip().replace(",", "-") if module in HOST_MODULES else ""
+    return os.path.join(_build_dir(), f"libphoton_{module}{'.' + tag if tag else ''}.so")
 
 
 def is_current(module: str) -> bool:
@@ -144,8 +168,8 @@ def build_module(module: str, force: bool = False, quiet: bool = False) -> str:
         return lib
     host = module in HOST_MODULES
     hipcc = _host_compiler() if host else _hipcc()
-    compile_flags = HOST_FLAGS if host else HIPCC_FLAGS
-    link_flags = ["-shared", "-fPIC"] if host else [f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc"]
+    compile_flags = HOST_FLAGS + sanitize_flags() if host else HIPCC_FLAGS
+    link_flags = ["-shared", "-fPIC"] + sanitize_flags() if host else [f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc"]
     link_libs: List[str] = []
     if module == "api":
         compile_flags = compile_flags + python_embed_flags()[0]

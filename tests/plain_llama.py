@@ -1,7 +1,7 @@
 """A plain, slow implementation of the Llama forward pass: whole sequences, no cache.
 
-Written from the reference's formulas (each function cites file:line under
-/root/reference); it shares no code with ``photon_infer_amd``.  Everything is explicit
+Written from the reference's formulas (each function cites file:line in the reference
+repository, lumia431/photon_infer); it shares no code with ``photon_infer_amd``.  Everything is explicit
 torch arithmetic on the CPU in float32 (or float64 when asked), one function per part.
 
 ``act_round`` lets a test emulate the places where the bfloat16 path rounds

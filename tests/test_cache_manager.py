@@ -149,3 +149,29 @@ def test_random_orders_never_lose_or_double_a_page(seed):
         m.release(rid)
     m.check_invariants()
     assert m.free_pages(0) == 24 and m.free_pages(1) == 12 and m.free_slots == 4
+
+
+def test_native_cache_manager_under_address_and_undefined_sanitizers(tmp_path):
+    """The host-side C++ of the cache manager, compiled whole with a random workload
+    (tests/cpp/cache_sanitize.cpp) under -fsanitize=address,undefined and run on the CPU: any
+    out-of-bounds access, use after free, leak or undefined operation ends it with a report."""
+    import os
+    import subprocess
+
+    from photon_infer_amd.errors import KernelLibraryMissing
+    from photon_infer_amd.ops import build
+
+    driver = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "cache_sanitize.cpp")
+    try:
+        exe = build.build_host_program([driver, "runtime/cache.cpp"], str(tmp_path / "cache_sanitize"), "address,undefined")
+    except KernelLibraryMissing as e:
+        if "sanitize" in str(e) or "asan" in str(e) or "ubsan" in str(e):
+            pytest.skip(f"this compiler has no sanitizer runtimes: {e}")
+        raise
+    env = dict(os.environ)
+    # the environment is left as it is: where it preloads libraries of its own, the sanitizer's
+    # runtime is not the first in the list, which it is told to accept
+    env["ASAN_OPTIONS"] = "detect_leaks=1:abort_on_error=0:verify_asan_link_order=0"
+    r = subprocess.run([exe, "60"], capture_output=True, text=True, timeout=300, env=env)
+    assert r.returncode == 0, r.stdout + r.stderr
+    assert r.stdout.strip() == "ok 60 seeds"
