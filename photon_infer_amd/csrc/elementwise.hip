@@ -120,10 +120,13 @@ __global__ void rmsnorm_wide_kernel(TO* __restrict__ out, float* __restrict__ x,
   }
   if (part) {
     const float* pr = part + r * D;
-    for (int s0 = 0; s0 < splits; s0 += 4) {     // four pieces' loads go out together, the adds keep the split order
-      float t[4][VPT][4];
+    // several pieces' loads go out together (eight where a thread holds few values: a decode
+    // step's eight pieces are then one wait for memory, not two); the adds keep the split order
+    constexpr int U = VPT <= 2 ? 8 : 4;
+    for (int s0 = 0; s0 < splits; s0 += U) {
+      float t[U][VPT][4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int k = 0; k < VPT; ++k) {
           const int gi = threadIdx.x + k * blockDim.x;
@@ -131,7 +134,7 @@ __global__ void rmsnorm_wide_kernel(TO* __restrict__ out, float* __restrict__ x,
           else t[u][k][0] = t[u][k][1] = t[u][k][2] = t[u][k][3] = 0.f;
         }
 #pragma unroll
-      for (int u = 0; u < 4; ++u)
+      for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int k = 0; k < VPT; ++k)
 #pragma unroll
