@@ -32,6 +32,8 @@ SHARED_FROM_TOKENS = 32        # more tokens than this: the skinny kernel that s
 SHARED_ROWS_PER_BLOCK = 64     # ... with this many weight rows per block ...
 SHARED_TARGET_BLOCKS = 256     # ... and this many blocks wanted (one per compute unit)
 TILE_MAX_SPLITS = 4
+BIG_MIN_TILES = 192            # 256 x 256 tiles (times k pieces) from which the large-tile kernel is taken (the library's rule)
+BIG_MIN_K = 1024               # a piece of the large-tile kernel keeps at least this much of k
 PIECES_BELOW_TILES = 200       # fewer 128 x 128 tiles than this: q, k, v of a prompt portion are left in k pieces too
 MAX_DECODE_SPLITS = 64         # the combine kernel holds one key range per lane
 DECODE_WAVES_WANTED = 512      # waves of the decode attention kernel that fill the chip (measured at batch 1 to 64: more is never faster)
@@ -58,7 +60,16 @@ def _skinny_splits(M: int, N: int, K: int) -> int:
 
 
 def _tile_splits(M: int, N: int, K: int) -> int:
-    """k-split of the tile kernel: only when its 128 x 128 tiles are too few to fill the chip."""
+    """k-split of the tile kernels: only when the output has too few tiles to fill the chip."""
+    big = -(-M // 256) * -(-N // 256)
+    if K % 64 == 0:
+        # a long k over few 256 x 256 tiles (the down projection of a 2,048-token prompt): as many
+        # pieces on the large-tile kernel as give every compute unit one block (measured at
+        # 2048 x 2048 x 8192: four pieces 72 us, against 87 us for two pieces on the small tiles,
+        # and 6 us more in the norm that adds them)
+        for pieces in (4, 3, 2):
+            if BIG_MIN_TILES <= big * pieces <= 256 and K >= pieces * BIG_MIN_K and pieces * M * N <= GEMM_PART_FLOATS:
+                return pieces
     tiles = -(-M // 128) * -(-N // 128)
     splits = min(TILE_MAX_SPLITS, TARGET_BLOCKS // max(1, tiles), K // 512)
     while splits > 1 and splits * M * N > GEMM_PART_FLOATS:
