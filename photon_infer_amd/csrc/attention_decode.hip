@@ -203,20 +203,22 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2
   // The wave whose keys end at the new token writes that token into the cache first and waits
   // for the stores; after that it reads the token like any other key, in the same order of
   // arithmetic as a kernel that finds the cache written: the same bits.
-  if (FUSED && src.write_kv && c0 < c1 && c1 == last_chunk + 1) {
-    store_new_kv<HD>(src, row, g, p, bt, table_width, nkv, page_size, num_pages, lane);
-    __threadfence_block();
+  if constexpr (FUSED) {
+    if (src.write_kv && c0 < c1 && c1 == last_chunk + 1) {
+      store_new_kv<HD>(src, row, g, p, bt, table_width, nkv, page_size, num_pages, lane);
+      __threadfence_block();
+    }
   }
   attn_walk<HD, 1>(st, c0, c1, (lo + 31) / 32, (p + 1) / 32 - 1, k_cache, v_cache, bt, table_width, kv_len, nkv, g,
                    page_size, num_pages, scale * PI_LOG2E, lane, [&]() {
                      // while the first keys and values are on their way
-                     if (!FUSED) {
+                     if constexpr (!FUSED) {
                        attn_load_q(st, 0, q, q_stride, row, g * G + lr, valid, lane);
-                       return;
+                     } else {
+                       const int none[1] = {0};
+                       float unused[1];
+                       rotated_fragments<HD, 0>(st.q[0], src, row, src.q_col + (g * G + lr) * HD, valid, lane, none, false, unused);
                      }
-                     const int none[1] = {0};
-                     float unused[1];
-                     rotated_fragments<HD, 0>(st.q[0], src, row, src.q_col + (g * G + lr) * HD, valid, lane, none, false, unused);
                    });
   attn_finish(st);
 
@@ -249,41 +251,43 @@ __global__ __launch_bounds__(64) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2
   }
 }
 
-// Merge the key ranges of one (request, head) by one wave: lane d owns feature d (and d + 64).
+// Merge the key ranges of one (request, head) by one wave: lane d owns features d, d + 64, ..
 // Ranges are added in range order; an empty range (m = -inf) counts nothing.
 template <int HD>
 __device__ inline void combine_ranges(bf16_t* __restrict__ o, const float* base, int splits, int lane) {
   const int rec = HD + 4;
+  constexpr int NF = (HD + 63) / 64;     // features per lane
   // lane s holds range s (splits <= 64): maxima, weights and the total in parallel
   const float ms = lane < splits ? base[lane * rec + HD] : -INFINITY;
   const float ls = lane < splits ? base[lane * rec + HD + 1] : 0.f;
   const float m_tot = wave_max(ms);
   const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - m_tot);   // maxima are in the base-2 scale
   float l_tot = 0.f;
-  float acc[HD / 64];
+  float acc[NF];
 #pragma unroll
-  for (int i = 0; i < HD / 64; ++i) acc[i] = 0.f;
+  for (int i = 0; i < NF; ++i) acc[i] = 0.f;
   // ranges in order; eight loads in flight at a time
   for (int s0 = 0; s0 < splits; s0 += 8) {
-    float ov[8][HD / 64], ws[8];
+    float ov[8][NF], ws[8];
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       const int s = s0 + u;
       ws[u] = __shfl(w, s < splits ? s : 0, 64);
       if (s >= splits) ws[u] = 0.f;
 #pragma unroll
-      for (int i = 0; i < HD / 64; ++i) ov[u][i] = (s < splits) ? base[s * rec + lane + i * 64] : 0.f;
+      for (int i = 0; i < NF; ++i) ov[u][i] = (s < splits && lane + i * 64 < HD) ? base[s * rec + lane + i * 64] : 0.f;
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
       l_tot += ws[u] * __shfl(ls, (s0 + u < splits) ? s0 + u : 0, 64);
 #pragma unroll
-      for (int i = 0; i < HD / 64; ++i) acc[i] += ws[u] * ov[u][i];
+      for (int i = 0; i < NF; ++i) acc[i] += ws[u] * ov[u][i];
     }
   }
   const float inv = 1.0f / l_tot;
 #pragma unroll
-  for (int i = 0; i < HD / 64; ++i) o[lane + i * 64] = from_float<bf16_t>(acc[i] * inv);
+  for (int i = 0; i < NF; ++i)
+    if (lane + i * 64 < HD) o[lane + i * 64] = from_float<bf16_t>(acc[i] * inv);
 }
 
 // One wave per (request, head).
@@ -301,6 +305,28 @@ __global__ __launch_bounds__(64) void attention_combine_kernel(bf16_t* __restric
                      splits, threadIdx.x);
 }
 
+// One wave per (row of `part`, head): rows are a launch's requests (results to the requests'
+// token rows) or listed token rows.
+static int launch_combine(void* out, long out_stride, const int* q_start, const int* req_ids, const int* rows, int Z,
+                          const void* part, int nh, int hd, int splits, hipStream_t stream) {
+  const dim3 grid(nh, Z), block(64);
+#define GO(H) hipLaunchKernelGGL(attention_combine_kernel<H>, grid, block, 0, stream, (bf16_t*)out, out_stride, q_start, req_ids, rows, \
+                                 (const float*)part, nh, splits)
+  switch (hd) {
+    case 32: GO(32); break;
+    case 64: GO(64); break;
+    case 96: GO(96); break;
+    case 128: GO(128); break;
+    case 160: GO(160); break;
+    case 192: GO(192); break;
+    case 224: GO(224); break;
+    case 256: GO(256); break;
+    default: return pi_fail("attention_combine: head_dim %d is not a multiple of 32 up to 256", hd);
+  }
+#undef GO
+  return pi_check_launch("attention_combine");
+}
+
 // part: float32 [R * nh * splits * (hd + 4)], needed when splits > 1.
 // req_ids: null (requests 0 .. R-1) or the R requests of the step that this launch serves; each
 // has one query token, at row q_start[r], that sees kv_len[r] keys.
@@ -310,7 +336,8 @@ static int launch_decode(bool fused, const DecodeSource& src, void* out, long ou
                          int page_size, float scale, int window, long num_pages, int splits, void* part, long part_elems,
                          hipStream_t stream) {
   PI_REQUIRE(R > 0 && nh > 0 && nkv > 0 && nh % nkv == 0 && nh / nkv <= 16, "attention_decode: needs 1..16 heads per kv head, got %d / %d", nh, nkv);
-  PI_REQUIRE(hd == 64 || hd == 128, "attention_decode: head_dim %d is not 64 or 128", hd);
+  PI_REQUIRE(hd >= 32 && hd <= 256 && hd % 32 == 0, "attention_decode: head_dim %d is not a multiple of 32 up to 256", hd);
+  PI_REQUIRE(!fused || hd == 64 || hd == 128, "attention_decode: the kernel that starts from the projection takes head_dim 64 or 128, not %d", hd);
   PI_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_decode: page size %d must be a multiple of 16", page_size);
   PI_REQUIRE(splits >= 1 && splits <= 64 && R <= 65535 && nkv <= 65535, "attention_decode: bad grid (%d ranges, %d requests, %d kv heads)", splits, R, nkv);
   PI_REQUIRE(out_stride % 4 == 0 && ((uintptr_t)out % 8 == 0), "attention_decode: out rows must be 8-byte aligned");
@@ -323,17 +350,21 @@ static int launch_decode(bool fused, const DecodeSource& src, void* out, long ou
                                     q_stride, src, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, \
                                     kv_len, req_ids, nh, nkv, page_size, scale, window, num_pages, (float*)part)
   if (fused) { if (hd == 64) GO(64, true); else GO(128, true); }
-  else { if (hd == 64) GO(64, false); else GO(128, false); }
+  else {
+    switch (hd) {
+      case 32: GO(32, false); break;
+      case 64: GO(64, false); break;
+      case 96: GO(96, false); break;
+      case 128: GO(128, false); break;
+      case 160: GO(160, false); break;
+      case 192: GO(192, false); break;
+      case 224: GO(224, false); break;
+      default: GO(256, false); break;
+    }
+  }
 #undef GO
   if (pi_check_launch("attention_decode")) return -1;
-  if (splits > 1) {
-    const dim3 cgrid(nh, R);
-    if (hd == 64)
-      hipLaunchKernelGGL(attention_combine_kernel<64>, cgrid, block, 0, stream, (bf16_t*)out, out_stride, q_start, req_ids, (const int*)nullptr, (const float*)part, nh, splits);
-    else
-      hipLaunchKernelGGL(attention_combine_kernel<128>, cgrid, block, 0, stream, (bf16_t*)out, out_stride, q_start, req_ids, (const int*)nullptr, (const float*)part, nh, splits);
-    return pi_check_launch("attention_combine");
-  }
+  if (splits > 1) return launch_combine(out, out_stride, q_start, req_ids, nullptr, R, part, nh, hd, splits, stream);
   return 0;
 }
 
@@ -392,13 +423,5 @@ extern "C" int pi_attention_decode_fused(void* out, long out_stride, const void*
 extern "C" int pi_attention_combine_rows(void* out, long out_stride, const int* rows, int Z, const void* part, int nh, int hd,
                                          int cuts, hipStream_t stream) {
   PI_REQUIRE(Z > 0 && Z <= 65535 && nh > 0 && cuts >= 2 && cuts <= 64 && rows && part, "attention_combine_rows: bad arguments (%d tokens, %d heads, %d cuts)", Z, nh, cuts);
-  PI_REQUIRE(hd == 64 || hd == 128, "attention_combine_rows: head_dim %d is not 64 or 128", hd);
-  const dim3 grid(nh, Z), block(64);
-  if (hd == 64)
-    hipLaunchKernelGGL(attention_combine_kernel<64>, grid, block, 0, stream, (bf16_t*)out, out_stride, (const int*)nullptr,
-                       (const int*)nullptr, rows, (const float*)part, nh, cuts);
-  else
-    hipLaunchKernelGGL(attention_combine_kernel<128>, grid, block, 0, stream, (bf16_t*)out, out_stride, (const int*)nullptr,
-                       (const int*)nullptr, rows, (const float*)part, nh, cuts);
-  return pi_check_launch("attention_combine_rows");
+  return launch_combine(out, out_stride, nullptr, nullptr, rows, Z, part, nh, hd, cuts, stream);
 }

@@ -200,7 +200,7 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
                                          int nkv, int hd, int page_size, float scale, int window, long num_pages,
                                          hipStream_t stream) {
   PI_REQUIRE(rounds > 0 && seats > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad sizes rounds=%d seats=%d heads=%d kv_heads=%d", rounds, seats, nh, nkv);
-  PI_REQUIRE(hd == 64 || hd == 128, "attention_prefill: head_dim %d is not 64 or 128", hd);
+  PI_REQUIRE(hd == 32 || hd == 64 || hd == 96 || hd == 128, "attention_prefill: head_dim %d is not 32, 64, 96 or 128", hd);
   PI_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_prefill: page size %d must be a multiple of 16", page_size);
   PI_REQUIRE(table_width >= 1, "attention_prefill: empty block table");
   const int TQ = pi_attention_tile_rows(nh, nkv, hd);
@@ -208,20 +208,25 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
   PI_REQUIRE(seats <= 65535, "attention_prefill: too many blocks per kv head (%d)", seats);
   PI_REQUIRE(out_stride % 4 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "attention_prefill: q / out rows must be 16- / 8-byte aligned");
   const size_t lds = tiles_lds_bytes(hd);
-  static bool configured[2] = {false, false};
-  if (!configured[hd == 128]) {
-    const void* fn = hd == 64 ? reinterpret_cast<const void*>(attention_tiles_kernel<64, 2>)
-                              : reinterpret_cast<const void*>(attention_tiles_kernel<128, 2>);
+  static bool configured[4] = {false, false, false, false};
+  if (!configured[hd / 32 - 1]) {
+    const void* fn = hd == 32   ? reinterpret_cast<const void*>(attention_tiles_kernel<32, 2>)
+                     : hd == 64 ? reinterpret_cast<const void*>(attention_tiles_kernel<64, 2>)
+                     : hd == 96 ? reinterpret_cast<const void*>(attention_tiles_kernel<96, 2>)
+                                : reinterpret_cast<const void*>(attention_tiles_kernel<128, 2>);
     hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return pi_fail("attention_prefill: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-    configured[hd == 128] = true;
+    configured[hd / 32 - 1] = true;
   }
   const dim3 grid(nkv, seats), block(256);
 #define GO(H, C) hipLaunchKernelGGL((attention_tiles_kernel<H, C>), grid, block, lds, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, \
                                     q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, \
                                     kv_len, tile_req, tile_q0, tile_cut, tile_z0, (float*)part, order, rounds, nh, nkv, page_size, scale, \
                                     window, num_pages, TQ)
-  if (hd == 64) GO(64, 2); else GO(128, 2);
+  if (hd == 32) GO(32, 2);
+  else if (hd == 64) GO(64, 2);
+  else if (hd == 96) GO(96, 2);
+  else GO(128, 2);
 #undef GO
   return pi_check_launch("attention_prefill_mfma");
 }

@@ -7,9 +7,10 @@ Which kernel takes what:
   * matrix products: K and the row strides multiples of 8, 16-byte aligned operands;
     up to 64 rows go to the weight-streaming kernel (k split over blocks where the output
     is narrow), more rows to the 128 x 128 tile kernel;
-  * attention: head_dim 64 or 128, pages of a multiple of 16 tokens; a batch of single
-    tokens with at most 16 heads per kv head goes to the key-split decode kernel, any other
-    batch to the tile kernel.
+  * attention: pages of a multiple of 16 tokens; a batch of single tokens with at most 16 heads
+    per kv head goes to the key-split decode kernel (head_dim a multiple of 32 up to 256; for
+    64 and 128 straight from the q|k|v projection), any other batch to the tile kernel
+    (head_dim 32, 64, 96, 128), its single tokens to the decode kernel.
 """
 from __future__ import annotations
 
@@ -35,6 +36,9 @@ TILE_MAX_SPLITS = 4
 BIG_MIN_TILES = 192            # 256 x 256 tiles (times k pieces) from which the large-tile kernel is taken (the library's rule)
 BIG_MIN_K = 1024               # a piece of the large-tile kernel keeps at least this much of k
 PIECES_BELOW_TILES = 200       # fewer 128 x 128 tiles than this: q, k, v of a prompt portion are left in k pieces too
+TILE_HEAD_DIMS = (32, 64, 96, 128)                 # head sizes of the prompt-attention tile kernel (its LDS holds two rounds of keys and values)
+DECODE_HEAD_DIMS = tuple(range(32, 257, 32))       # head sizes of the key-split decode kernel
+FUSED_DECODE_HEAD_DIMS = (64, 128)                 # ... and of its form that starts from the q|k|v projection (whole halves of a head per fragment)
 MAX_DECODE_SPLITS = 64         # the combine kernel holds one key range per lane
 DECODE_WAVES_WANTED = 512      # waves of the decode attention kernel that fill the chip (measured at batch 1 to 64: more is never faster)
 DECODE_MIN_KEYS_PER_SPLIT = 128
@@ -287,7 +291,7 @@ class AttentionPlanner:
 def attention_planner(dtype, num_heads: int, num_kv_heads: int, head_dim: int, page_size: int, window: int,
                       device) -> Optional[AttentionPlanner]:
     """The planner for a mixer of these sizes, or None when the general kernel serves it."""
-    if dtype != torch.bfloat16 or head_dim not in (64, 128) or page_size % 16:
+    if dtype != torch.bfloat16 or head_dim not in TILE_HEAD_DIMS or page_size % 16:
         return None
     tile_rows = attention_tile_rows(num_heads, num_kv_heads, head_dim)
     if tile_rows < 1:
@@ -388,7 +392,7 @@ def _decode_splits_that_fit(ws, n_req: int, num_heads: int, num_kv_heads: int, h
 
 def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
                     page_size, scale, window, pages, ws: Optional[KernelWorkspace] = None) -> bool:
-    if head_dim not in (64, 128) or page_size % 16 or q.data_ptr() % 16 or q.stride(0) % 8 or out.stride(0) % 4:
+    if head_dim not in DECODE_HEAD_DIMS or page_size % 16 or q.data_ptr() % 16 or q.stride(0) % 8 or out.stride(0) % 4:
         return False
     G = num_heads // num_kv_heads
     R = ctx.R
@@ -433,7 +437,7 @@ def decode_attention_from_projection(out, qkv, ctx, table, num_heads, num_kv_hea
     tensor [T, N] or ``Partials``), which the kernel rotates by ``table`` (the step's cos / sin
     table [T, head_dim], or None) and whose keys and values it stores.  False: not for these sizes."""
     G = num_heads // num_kv_heads
-    if not ctx.all_decode or G > 16 or head_dim not in (64, 128) or page_size % 16 or out.stride(0) % 4:
+    if not ctx.all_decode or G > 16 or head_dim not in FUSED_DECODE_HEAD_DIMS or page_size % 16 or out.stride(0) % 4:
         return False
     R = ctx.R
     pieces = isinstance(qkv, Partials)

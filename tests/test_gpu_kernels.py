@@ -518,6 +518,16 @@ ATTN_CASES = [
     (8, 2, 64, 64, [130, 3, 1], [130, 250, 99], 33),                 # portions with a window, pages of 64
     (16, 1, 64, 16, [1, 1], [129, 2], None),                         # sixteen heads on one kv head
     (32, 1, 64, 16, [1, 70], [75, 70], None),                        # more heads per kv head than a wave's columns
+    # the other head sizes of the matrix-core kernels: 32 and 96 (tile and decode kernel), 160 .. 256 (decode kernel)
+    (4, 2, 32, 16, [1, 1, 1], [5, 100, 333], None),
+    (4, 2, 32, 16, [70, 1, 3], [300, 20, 64], None),
+    (6, 2, 96, 16, [40, 1, 2, 100], [40, 77, 300, 100], None),
+    (3, 3, 96, 32, [1, 1, 1, 1], [1, 32, 33, 500], 48),
+    (4, 2, 160, 32, [1, 1], [129, 64], None),
+    (4, 1, 192, 16, [1, 1], [50, 700], None),
+    (8, 2, 224, 16, [1], [300], 100),
+    (2, 2, 256, 16, [1, 1, 1], [1, 33, 400], None),
+    (4, 1, 192, 16, [5, 1], [50, 700], None),                        # a portion at a head size the tile kernel does not take
     (8, 2, 128, 16, [1, 70, 1, 1, 2], [900, 300, 33, 1, 50], None),  # single tokens beside portions: two kernels share the step
     (4, 2, 64, 16, [1, 3, 1], [700, 40, 18], 25),                    # the same with a window
     (8, 2, 64, 16, [70, 5], [2100, 40], None),                       # few tiles, many keys: their key ranges are cut and merged

@@ -72,8 +72,19 @@ TINY_F = dict(
 )
 TINY_F_INIT = dict(std=0.03, norm_init="uniform", block_size=16)
 
+# a head size of 96: three fragments of 32 features in the matrix-core attention kernels (tile
+# kernel and key-split decode kernel; the decode kernel that starts from the projection takes
+# 64 and 128 only, so single tokens go through the separate rotation kernel)
+TINY_G = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=160, intermediate_size=264, num_hidden_layers=2,
+    num_attention_heads=3, num_key_value_heads=1, head_dim=96, vocab_size=600, max_position_embeddings=512,
+    rms_norm_eps=1e-5, rope_theta=20000.0, tie_word_embeddings=True,
+)
+TINY_G_INIT = dict(std=0.07, norm_init="uniform", block_size=16)
+
 ALL = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT), "D": (TINY_D, TINY_D_INIT),
-       "E": (TINY_E, TINY_E_INIT), "F": (TINY_F, TINY_F_INIT)}
+       "E": (TINY_E, TINY_E_INIT), "F": (TINY_F, TINY_F_INIT),
+       "G": (TINY_G, TINY_G_INIT)}
 
 
 def make_model_dir(tmp_path, name: str, seed: int = 0, storage: str = "bfloat16") -> str:
