@@ -313,15 +313,23 @@ static int launch_combine(void* out, long out_stride, const int* q_start, const 
 #define GO(H) hipLaunchKernelGGL(attention_combine_kernel<H>, grid, block, 0, stream, (bf16_t*)out, out_stride, q_start, req_ids, rows, \
                                  (const float*)part, nh, splits)
   switch (hd) {
+    case 16: GO(16); break;
     case 32: GO(32); break;
+    case 48: GO(48); break;
     case 64: GO(64); break;
+    case 80: GO(80); break;
     case 96: GO(96); break;
+    case 112: GO(112); break;
     case 128: GO(128); break;
+    case 144: GO(144); break;
     case 160: GO(160); break;
+    case 176: GO(176); break;
     case 192: GO(192); break;
+    case 208: GO(208); break;
     case 224: GO(224); break;
+    case 240: GO(240); break;
     case 256: GO(256); break;
-    default: return pi_fail("attention_combine: head_dim %d is not a multiple of 32 up to 256", hd);
+    default: return pi_fail("attention_combine: head_dim %d is not a multiple of 16 up to 256", hd);
   }
 #undef GO
   return pi_check_launch("attention_combine");
@@ -336,7 +344,7 @@ static int launch_decode(bool fused, const DecodeSource& src, void* out, long ou
                          int page_size, float scale, int window, long num_pages, int splits, void* part, long part_elems,
                          hipStream_t stream) {
   PI_REQUIRE(R > 0 && nh > 0 && nkv > 0 && nh % nkv == 0 && nh / nkv <= 16, "attention_decode: needs 1..16 heads per kv head, got %d / %d", nh, nkv);
-  PI_REQUIRE(hd >= 32 && hd <= 256 && hd % 32 == 0, "attention_decode: head_dim %d is not a multiple of 32 up to 256", hd);
+  PI_REQUIRE(hd >= 16 && hd <= 256 && hd % 16 == 0, "attention_decode: head_dim %d is not a multiple of 16 up to 256", hd);
   PI_REQUIRE(!fused || hd == 64 || hd == 128, "attention_decode: the kernel that starts from the projection takes head_dim 64 or 128, not %d", hd);
   PI_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_decode: page size %d must be a multiple of 16", page_size);
   PI_REQUIRE(splits >= 1 && splits <= 64 && R <= 65535 && nkv <= 65535, "attention_decode: bad grid (%d ranges, %d requests, %d kv heads)", splits, R, nkv);
@@ -352,13 +360,21 @@ static int launch_decode(bool fused, const DecodeSource& src, void* out, long ou
   if (fused) { if (hd == 64) GO(64, true); else GO(128, true); }
   else {
     switch (hd) {
+      case 16: GO(16, false); break;
       case 32: GO(32, false); break;
+      case 48: GO(48, false); break;
       case 64: GO(64, false); break;
+      case 80: GO(80, false); break;
       case 96: GO(96, false); break;
+      case 112: GO(112, false); break;
       case 128: GO(128, false); break;
+      case 144: GO(144, false); break;
       case 160: GO(160, false); break;
+      case 176: GO(176, false); break;
       case 192: GO(192, false); break;
+      case 208: GO(208, false); break;
       case 224: GO(224, false); break;
+      case 240: GO(240, false); break;
       default: GO(256, false); break;
     }
   }

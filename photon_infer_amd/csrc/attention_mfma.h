@@ -24,9 +24,18 @@
 
 #define PI_LOG2E 1.4426950408889634f
 
+// A head of HD features (a multiple of 16) is contracted in KS fragments of 32; when HD is no
+// multiple of 32 the upper half of the last fragment (the lanes of groups 2 and 3) is zero in
+// the queries and in the keys.
+template <int HD>
+struct HeadFrags {
+  static constexpr int KS = (HD + 31) / 32;
+  __device__ static inline bool holds(int ks, int lane) { return ks * 32 + (lane / 16) * 8 < HD; }   // false only in a half fragment
+};
+
 template <int HD, int CB>
 struct AttnState {
-  Frag q[CB][HD / 32];
+  Frag q[CB][HeadFrags<HD>::KS];
   f32x4_t o[HD / 16][CB];
   float m[CB];          // reference score of the column (raw units, see attn_compute)
   f32x4_t ls[CB];       // the column's sum of weights, four times over (see weight_sum)
@@ -37,7 +46,7 @@ struct AttnState {
 
 template <int HD>
 struct KVChunk {
-  Frag k[2][HD / 32];   // key tiles: rows key0 + lane % 16
+  Frag k[2][HeadFrags<HD>::KS];   // key tiles: rows key0 + lane % 16
   Frag v[HD / 16];      // value rows d = db*16 + lane % 16; keys (lane/16)*4..+3 of both tiles
   bool have[2];
   __device__ inline Frag key(int t, int ks) const { return k[t][ks]; }
@@ -50,8 +59,8 @@ template <int HD>
 struct StagedChunk {
   const u32x4_t* from;  // this lane's first fragment
   bool have[2];
-  __device__ inline Frag key(int t, int ks) const { Frag f; f.n = from[(t * (HD / 32) + ks) * 64]; return f; }
-  __device__ inline Frag val(int db) const { Frag f; f.n = from[(HD / 16 + db) * 64]; return f; }
+  __device__ inline Frag key(int t, int ks) const { Frag f; f.n = from[(t * HeadFrags<HD>::KS + ks) * 64]; return f; }
+  __device__ inline Frag val(int db) const { Frag f; f.n = from[(2 * HeadFrags<HD>::KS + db) * 64]; return f; }
 };
 
 template <int HD, int CB>
@@ -131,10 +140,14 @@ struct PageCursor {
 template <int HD>
 struct KVLaneOffsets {
   uint32_t k;              // key row lane % 16, features (lane / 16) * 8 ..
+  uint32_t k0;             // the row's first features (what a lane without features of its own reads)
+  bool tail;               // the lane holds features of the last fragment (always, unless HD % 32 == 16)
   uint32_t v[HD / 16];     // value row db * 16 + lane % 16, keys (lane / 16) * 4 ..
   __device__ inline void set(int page_size, int lane) {
     const int lr = lane % 16, lg = lane / 16;
     k = (uint32_t)(lr * HD + lg * 8) * 2u;
+    k0 = (uint32_t)(lr * HD) * 2u;
+    tail = HeadFrags<HD>::holds(HeadFrags<HD>::KS - 1, lane);
 #pragma unroll
     for (int db = 0; db < HD / 16; ++db) v[db] = (uint32_t)((db * 16 + lr) * page_size + lg * 4) * 2u;
   }
@@ -156,7 +169,12 @@ __device__ inline void attn_load(KVChunk<HD>& kv, const ChunkPages& cp, const bf
     const char* kp = reinterpret_cast<const char*>(k_cache + pg * page_elems + (long)(g * page_size + cp.slot[t]) * HD);
     const char* vp = reinterpret_cast<const char*>(v_cache + pg * page_elems + (long)g * page_size * HD + cp.slot[t]);
 #pragma unroll
-    for (int ks = 0; ks < HD / 32; ++ks) kv.k[t][ks].n = *reinterpret_cast<const u32x4_t*>(kp + off.k + ks * 64);
+    for (int ks = 0; ks < HeadFrags<HD>::KS; ++ks) {
+      // a half fragment's upper lanes read their row's first features again and count as zero
+      const bool held = HD % 32 == 0 || ks + 1 < HeadFrags<HD>::KS || off.tail;
+      kv.k[t][ks].n = *reinterpret_cast<const u32x4_t*>(kp + (held ? off.k + ks * 64 : off.k0));
+      if (!held) kv.k[t][ks].n = u32x4_t{0u, 0u, 0u, 0u};
+    }
 #pragma unroll
     for (int db = 0; db < HD / 16; ++db) kv.v[db].d[t] = *reinterpret_cast<const uint2*>(vp + off.v[db]);
   }
@@ -182,7 +200,7 @@ __device__ inline void attn_compute(AttnState<HD, CB>& st, const KV& kv, int k0,
     for (int c = 0; c < CB; ++c) {
       f32x4_t acc = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < HD / 32; ++ks) acc = mfma16(kv.key(t, ks), st.q[c][ks], acc);
+      for (int ks = 0; ks < HeadFrags<HD>::KS; ++ks) acc = mfma16(kv.key(t, ks), st.q[c][ks], acc);
       s[t][c] = acc;
     }
   const float slack = PI_RESCALE_SLACK / scale_log2;
@@ -261,7 +279,8 @@ __device__ inline void attn_compute_plain(AttnState<HD, CB>& st, const u32x4_t* 
   // The key fragments of a chunk are read from LDS while the products of the chunk before it
   // run; the scheduler is told so, or it reads each fragment right before its use to save
   // registers and the wave waits for LDS sixteen times per group.
-  constexpr int KF = 2 * (HD / 32);
+  constexpr int KS = HeadFrags<HD>::KS;
+  constexpr int KF = 2 * KS;
   Frag kf[2][KF];
   f32x4_t s[NJ][2][CB];
 #pragma unroll
@@ -277,9 +296,9 @@ __device__ inline void attn_compute_plain(AttnState<HD, CB>& st, const u32x4_t* 
 #pragma unroll
       for (int c = 0; c < CB; ++c) s[j][t][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-      for (int ks = 0; ks < HD / 32; ++ks)
+      for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-        for (int c = 0; c < CB; ++c) s[j][t][c] = mfma16(kf[j & 1][t * (HD / 32) + ks], st.q[c][ks], s[j][t][c]);
+        for (int c = 0; c < CB; ++c) s[j][t][c] = mfma16(kf[j & 1][t * KS + ks], st.q[c][ks], s[j][t][c]);
     }
     if (j + 1 < NJ) __builtin_amdgcn_sched_group_barrier(0x100, KF, 0);   // LDS reads of the next chunk
     __builtin_amdgcn_sched_group_barrier(0x008, KF * CB, 0);               // this chunk's products
@@ -306,7 +325,7 @@ __device__ inline void attn_compute_plain(AttnState<HD, CB>& st, const u32x4_t* 
     for (int j = 0; j < NJ; ++j) {
       Frag va[HD / 16];
 #pragma unroll
-      for (int db = 0; db < HD / 16; ++db) va[db].n = from[j * chunk_stride + (HD / 16 + db) * 64];
+      for (int db = 0; db < HD / 16; ++db) va[db].n = from[j * chunk_stride + (KF + db) * 64];
 #pragma unroll
       for (int c = 0; c < CB; ++c) {
         float p[2][4];
@@ -402,7 +421,8 @@ __device__ inline void attn_load_q(AttnState<HD, CB>& st, int c, const bf16_t* _
                                    int head, bool valid, int lane) {
   const int lg = lane / 16;
 #pragma unroll
-  for (int ks = 0; ks < HD / 32; ++ks)
-    st.q[c][ks].n = valid ? *reinterpret_cast<const u32x4_t*>(q + row * q_stride + (long)head * HD + ks * 32 + lg * 8)
-                          : u32x4_t{0u, 0u, 0u, 0u};
+  for (int ks = 0; ks < HeadFrags<HD>::KS; ++ks)
+    st.q[c][ks].n = (valid && HeadFrags<HD>::holds(ks, lane))
+                        ? *reinterpret_cast<const u32x4_t*>(q + row * q_stride + (long)head * HD + ks * 32 + lg * 8)
+                        : u32x4_t{0u, 0u, 0u, 0u};
 }

@@ -28,7 +28,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
     const int* __restrict__ tile_req, const int* __restrict__ tile_q0, const int* __restrict__ tile_cut,
     const int* __restrict__ tile_z0, float* __restrict__ part, const int* __restrict__ order, int rounds, int nh,
     int nkv, int page_size, float scale, int window, long num_pages_l, int TQ) {
-  constexpr int F = HD / 8;                       // 16-byte operand fragments per lane and 32 keys: keys HD/16, values HD/16
+  constexpr int KS = HeadFrags<HD>::KS;
+  constexpr int F = 2 * KS + HD / 16;             // 16-byte operand fragments per lane and 32 keys: keys, then values
   extern __shared__ __attribute__((aligned(16))) u32x4_t staged[];   // [2 buffers][4 chunks][F][64 lanes]
   __shared__ int present[2][4][2];                // is the page of a 16-key tile there
   const int lane = threadIdx.x % 64;
@@ -107,10 +108,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
-        for (int ks = 0; ks < HD / 32; ++ks) mine[(t * (HD / 32) + ks) * 64] = pre.k[t][ks].n;
+        for (int ks = 0; ks < KS; ++ks) mine[(t * KS + ks) * 64] = pre.k[t][ks].n;
 #pragma unroll
       for (int db = 0; db < HD / 16; ++db)
-        mine[(HD / 16 + db) * 64] = u32x4_t{pre.v[db].d[0].x, pre.v[db].d[0].y, pre.v[db].d[1].x, pre.v[db].d[1].y};
+        mine[(2 * KS + db) * 64] = u32x4_t{pre.v[db].d[0].x, pre.v[db].d[0].y, pre.v[db].d[1].x, pre.v[db].d[1].y};
       if (lane < 2) present[buf][wave][lane] = lane == 0 ? pre.have[0] : pre.have[1];
     };
 
@@ -187,7 +188,7 @@ extern "C" int pi_attention_tile_rows(int nh, int nkv, int hd) {
 }
 
 // Shared memory of one block: two buffers of 128 keys and their values.
-static size_t tiles_lds_bytes(int hd) { return (size_t)2 * 4 * (hd / 8) * 64 * 16; }
+static size_t tiles_lds_bytes(int hd) { return (size_t)2 * 4 * (2 * ((hd + 31) / 32) + hd / 16) * 64 * 16; }
 
 // `order`: [rounds, seats] tile indices (-1: none), the host's deal of the tiles to `seats`
 // blocks per kv head.  tile_cut[t] = cut | cuts << 8: which of how many shares of its keys entry
@@ -200,7 +201,7 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
                                          int nkv, int hd, int page_size, float scale, int window, long num_pages,
                                          hipStream_t stream) {
   PI_REQUIRE(rounds > 0 && seats > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad sizes rounds=%d seats=%d heads=%d kv_heads=%d", rounds, seats, nh, nkv);
-  PI_REQUIRE(hd == 32 || hd == 64 || hd == 96 || hd == 128, "attention_prefill: head_dim %d is not 32, 64, 96 or 128", hd);
+  PI_REQUIRE(hd >= 16 && hd <= 128 && hd % 16 == 0, "attention_prefill: head_dim %d is not a multiple of 16 up to 128", hd);
   PI_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_prefill: page size %d must be a multiple of 16", page_size);
   PI_REQUIRE(table_width >= 1, "attention_prefill: empty block table");
   const int TQ = pi_attention_tile_rows(nh, nkv, hd);
@@ -208,25 +209,30 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
   PI_REQUIRE(seats <= 65535, "attention_prefill: too many blocks per kv head (%d)", seats);
   PI_REQUIRE(out_stride % 4 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "attention_prefill: q / out rows must be 16- / 8-byte aligned");
   const size_t lds = tiles_lds_bytes(hd);
-  static bool configured[4] = {false, false, false, false};
-  if (!configured[hd / 32 - 1]) {
-    const void* fn = hd == 32   ? reinterpret_cast<const void*>(attention_tiles_kernel<32, 2>)
-                     : hd == 64 ? reinterpret_cast<const void*>(attention_tiles_kernel<64, 2>)
-                     : hd == 96 ? reinterpret_cast<const void*>(attention_tiles_kernel<96, 2>)
-                                : reinterpret_cast<const void*>(attention_tiles_kernel<128, 2>);
-    hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    if (e != hipSuccess) return pi_fail("attention_prefill: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));
-    configured[hd / 32 - 1] = true;
-  }
   const dim3 grid(nkv, seats), block(256);
-#define GO(H, C) hipLaunchKernelGGL((attention_tiles_kernel<H, C>), grid, block, lds, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, \
-                                    q_stride, (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, \
-                                    kv_len, tile_req, tile_q0, tile_cut, tile_z0, (float*)part, order, rounds, nh, nkv, page_size, scale, \
-                                    window, num_pages, TQ)
-  if (hd == 32) GO(32, 2);
-  else if (hd == 64) GO(64, 2);
-  else if (hd == 96) GO(96, 2);
-  else GO(128, 2);
+#define GO(H, C)                                                                                                                           \
+  do {                                                                                                                                     \
+    static bool configured = false;                                                                                                        \
+    if (!configured) {                                                                                                                     \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_tiles_kernel<H, C>),                                      \
+                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                                            \
+      if (e != hipSuccess) return pi_fail("attention_prefill: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));            \
+      configured = true;                                                                                                                   \
+    }                                                                                                                                      \
+    hipLaunchKernelGGL((attention_tiles_kernel<H, C>), grid, block, lds, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride,     \
+                       (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, kv_len, tile_req, tile_q0,       \
+                       tile_cut, tile_z0, (float*)part, order, rounds, nh, nkv, page_size, scale, window, num_pages, TQ);                  \
+  } while (0)
+  switch (hd) {
+    case 16: GO(16, 2); break;
+    case 32: GO(32, 2); break;
+    case 48: GO(48, 2); break;
+    case 64: GO(64, 2); break;
+    case 80: GO(80, 2); break;
+    case 96: GO(96, 2); break;
+    case 112: GO(112, 2); break;
+    default: GO(128, 2); break;
+  }
 #undef GO
   return pi_check_launch("attention_prefill_mfma");
 }

@@ -8,9 +8,9 @@ Which kernel takes what:
     up to 64 rows go to the weight-streaming kernel (k split over blocks where the output
     is narrow), more rows to the 128 x 128 tile kernel;
   * attention: pages of a multiple of 16 tokens; a batch of single tokens with at most 16 heads
-    per kv head goes to the key-split decode kernel (head_dim a multiple of 32 up to 256; for
+    per kv head goes to the key-split decode kernel (head_dim a multiple of 16 up to 256; for
     64 and 128 straight from the q|k|v projection), any other batch to the tile kernel
-    (head_dim 32, 64, 96, 128), its single tokens to the decode kernel.
+    (head_dim a multiple of 16 up to 128), its single tokens to the decode kernel.
 """
 from __future__ import annotations
 
@@ -36,8 +36,8 @@ TILE_MAX_SPLITS = 4
 BIG_MIN_TILES = 192            # 256 x 256 tiles (times k pieces) from which the large-tile kernel is taken (the library's rule)
 BIG_MIN_K = 1024               # a piece of the large-tile kernel keeps at least this much of k
 PIECES_BELOW_TILES = 200       # fewer 128 x 128 tiles than this: q, k, v of a prompt portion are left in k pieces too
-TILE_HEAD_DIMS = (32, 64, 96, 128)                 # head sizes of the prompt-attention tile kernel (its LDS holds two rounds of keys and values)
-DECODE_HEAD_DIMS = tuple(range(32, 257, 32))       # head sizes of the key-split decode kernel
+TILE_HEAD_DIMS = tuple(range(16, 129, 16))         # head sizes of the prompt-attention tile kernel (its LDS holds two rounds of keys and values)
+DECODE_HEAD_DIMS = tuple(range(16, 257, 16))       # head sizes of the key-split decode kernel
 FUSED_DECODE_HEAD_DIMS = (64, 128)                 # ... and of its form that starts from the q|k|v projection (whole halves of a head per fragment)
 MAX_DECODE_SPLITS = 64         # the combine kernel holds one key range per lane
 DECODE_WAVES_WANTED = 512      # waves of the decode attention kernel that fill the chip (measured at batch 1 to 64: more is never faster)

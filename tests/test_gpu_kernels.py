@@ -518,7 +518,16 @@ ATTN_CASES = [
     (8, 2, 64, 64, [130, 3, 1], [130, 250, 99], 33),                 # portions with a window, pages of 64
     (16, 1, 64, 16, [1, 1], [129, 2], None),                         # sixteen heads on one kv head
     (32, 1, 64, 16, [1, 70], [75, 70], None),                        # more heads per kv head than a wave's columns
-    # the other head sizes of the matrix-core kernels: 32 and 96 (tile and decode kernel), 160 .. 256 (decode kernel)
+    # the other head sizes of the matrix-core kernels: every multiple of 16 up to 128 (tile and decode
+    # kernel) and up to 256 (decode kernel); sizes that are no multiple of 32 end in half a fragment
+    (4, 2, 16, 16, [1, 20, 1], [40, 20, 300], None),
+    (3, 1, 48, 16, [33, 1, 2], [33, 90, 130], None),
+    (4, 4, 80, 16, [1, 5, 1], [90, 37, 600], 16),
+    (5, 5, 80, 32, [64, 1], [200, 257], None),
+    (2, 1, 112, 16, [1, 1, 17], [15, 129, 50], None),
+    (2, 2, 144, 16, [1, 1], [100, 31], None),
+    (4, 2, 176, 16, [1], [260], None),
+    (3, 1, 240, 16, [1, 1], [64, 65], 30),
     (4, 2, 32, 16, [1, 1, 1], [5, 100, 333], None),
     (4, 2, 32, 16, [70, 1, 3], [300, 20, 64], None),
     (6, 2, 96, 16, [40, 1, 2, 100], [40, 77, 300, 100], None),
