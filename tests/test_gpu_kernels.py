@@ -607,6 +607,98 @@ def test_attention_finds_one_far_key_among_hundreds(_ops, dtype, fast):
                 assert (out[t] - want).abs().max() < 0.05
 
 
+def test_pages_beyond_four_gibibytes_of_a_pool(_ops):
+    """A pool of keys (and one of values) larger than 2^32 bytes, the requests' pages at its far
+    end and a few at its start: the rotation's cache write, both prompt kernels, the decode
+    kernel and the one that starts from the projection address them right.  A page id times a
+    page's bytes that was formed in 32 bits would read the fill (1e4) or write somewhere else,
+    which the count of changed cells shows."""
+    nh, nkv, hd, page, dtype = 16, 8, 128, 16, BF16
+    page_bytes = nkv * page * hd * 2
+    pages = (1 << 32) // page_bytes + 3000
+    q_lens, kv_lens = [40, 1, 1, 23], [40, 700, 33, 300]
+    R, T = len(q_lens), sum(q_lens)
+    g = gen(5)
+    seqs = [((torch.randn(kv, nkv, hd, generator=g) * 0.5).to(dtype), torch.randn(kv, nkv, hd, generator=g).to(dtype)) for kv in kv_lens]
+    blocks = [-(-kv // page) for kv in kv_lens]
+    ids = torch.randperm(2900, generator=g)[:sum(blocks)] + (pages - 2900)          # beyond 4 GiB
+    ids[::7] = torch.randperm(1000, generator=g)[:len(ids[::7])]                   # and some at the start
+    table = torch.full((R, max(blocks)), -1, dtype=torch.int32)
+    kc = torch.full((pages, nkv, page, hd), 1e4, dtype=dtype, device=DEV)
+    vc = torch.full((pages, nkv, hd, page), -1e4, dtype=dtype, device=DEV)
+    assert kc.numel() * 2 > 1 << 32
+    it = iter(ids.tolist())
+    old_cells = 0
+    for r, (k, v) in enumerate(seqs):
+        old = kv_lens[r] - q_lens[r]                       # what earlier steps left; this step's tokens come through the kernels
+        for b in range(blocks[r]):
+            pg = next(it)
+            table[r, b] = pg
+            n = max(0, min(page, old - b * page))
+            if n:
+                kc[pg, :, :n] = k[b * page: b * page + n].transpose(0, 1).to(DEV)
+                vc[pg, :, :, :n] = v[b * page: b * page + n].permute(1, 2, 0).to(DEV)
+            old_cells += n
+    table_d = table.to(DEV)
+    ctx = attention_ctx(q_lens, kv_lens, dtype)
+    freqs = P.rope_frequencies(hd, 10000.0, None)
+    inv = torch.tensor(freqs, dtype=torch.float64).to(F32).to(DEV)
+    pos = ctx.positions.cpu().tolist()
+    # this step's tokens: q, k, v before the rotation, such that the rotated keys are the sequences' own
+    new_k = torch.cat([k[kv - n:] for (k, _), n, kv in zip(seqs, q_lens, kv_lens)]).float()
+    new_v = torch.cat([v[kv - n:] for (_, v), n, kv in zip(seqs, q_lens, kv_lens)]).float()
+    q_raw = (torch.randn(T, nh, hd, generator=g) * 2).to(dtype)
+    qkv = torch.cat([q_raw.reshape(T, -1), new_k.to(dtype).reshape(T, -1), new_v.to(dtype).reshape(T, -1)], dim=1).to(DEV)
+    q = qkv[:, :nh * hd]
+    _ops.rope_kv_write(q, qkv[:, nh * hd:(nh + nkv) * hd], qkv[:, (nh + nkv) * hd:], ctx.positions, ctx.req_of_token, (inv, hd, False),
+                       nh, nkv, hd, kc, vc, table_d, page)
+    fill = torch.tensor(1e4, dtype=dtype).item()          # the fill as bfloat16 holds it
+    changed_k = int((kc != fill).sum().item())
+    changed_v = int((vc != -fill).sum().item())
+    assert changed_k == changed_v == (old_cells + T) * nkv * hd, "cells were written elsewhere, or not at all"
+    k_rot = P.rope(new_k, pos, freqs, False)
+    req = ctx.req_of_token.cpu().tolist()
+    for t in (0, 39, 40, 41, 42, T - 1):
+        pg, sl = table[req[t], pos[t] // page].item(), pos[t] % page
+        close(kc[pg, :, sl], k_rot[t], 2 ** -8, f"k of token {t}")
+        assert torch.equal(vc[pg, :, :, sl].cpu().float(), new_v[t].to(dtype).float())
+    # attention over what the cache now holds, by every kernel
+    dense, row = [], 0
+    for r, kv in enumerate(kv_lens):
+        pgs = table[r, :blocks[r]].tolist()
+        dense.append((torch.cat([kc[pg].transpose(0, 1) for pg in pgs])[:kv].cpu().float(),
+                      torch.cat([vc[pg].permute(2, 0, 1) for pg in pgs])[:kv].cpu().float()))
+    qs, row = [], 0
+    for n in q_lens:
+        qs.append(q[row:row + n].cpu().float().reshape(n, nh, hd))
+        row += n
+    scale = hd ** -0.5
+    want = dense_attention(qs, dense, q_lens, kv_lens, scale, None).reshape(T, nh * hd)
+    for fast in (True, False):
+        _ops.use_fast_kernels(fast)
+        out = torch.empty(T, nh * hd, dtype=dtype, device=DEV)
+        _ops.paged_attention(out, q.contiguous(), kc, vc, table_d, ctx, nh, nkv, hd, page, scale, 0)
+        close(out, want, 2 ** -7, f"attention, matrix-core kernels {fast}")
+    _ops.use_fast_kernels(True)
+    # a step of single tokens through the kernel that starts from the projection
+    ctx1 = attention_ctx([1] * R, [kv + 1 for kv in kv_lens], dtype)
+    assert all(kv % page for kv in kv_lens)       # every request's last page has room for one more token
+    step = (torch.randn(R, (nh + 2 * nkv) * hd, generator=g) * 0.6).to(dtype).to(DEV)
+    got = torch.empty(R, nh * hd, dtype=dtype, device=DEV)
+    assert _ops.decode_attention_from_projection(got, step, ctx1, (inv, hd, False), nh, nkv, hd, kc, vc, table_d, page, scale, 0, True)
+    assert int((kc != fill).sum().item()) == changed_k + R * nkv * hd
+    dense1, q1 = [], []
+    pos1 = ctx1.positions.cpu().tolist()
+    q_rot = P.rope(step[:, :nh * hd].cpu().float().reshape(R, nh, hd), pos1, freqs, False).to(dtype).float()
+    for r, kv in enumerate(kv_lens):
+        pgs = table[r, :-(-(kv + 1) // page)].tolist()
+        dense1.append((torch.cat([kc[pg].transpose(0, 1) for pg in pgs])[:kv + 1].cpu().float(),
+                       torch.cat([vc[pg].permute(2, 0, 1) for pg in pgs])[:kv + 1].cpu().float()))
+        q1.append(q_rot[r:r + 1])
+    want1 = dense_attention(q1, dense1, [1] * R, [kv + 1 for kv in kv_lens], scale, None).reshape(R, nh * hd)
+    close(got, want1, 2 ** -7, "from the projection")
+
+
 # ------------------------------------------------------------------ sampling
 def test_greedy_takes_the_lowest_index_among_equals(_ops):
     V = 128256
