@@ -261,7 +261,7 @@ __device__ inline void combine_ranges(bf16_t* __restrict__ o, const float* base,
   const float ms = lane < splits ? base[lane * rec + HD] : -INFINITY;
   const float ls = lane < splits ? base[lane * rec + HD + 1] : 0.f;
   const float m_tot = wave_max(ms);
-  const float w = (ms == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(ms - m_tot);   // maxima are in the base-2 scale
+  const float w = range_weight(ms, m_tot);
   float l_tot = 0.f;
   float acc[NF];
 #pragma unroll
@@ -279,15 +279,14 @@ __device__ inline void combine_ranges(bf16_t* __restrict__ o, const float* base,
     }
 #pragma unroll
     for (int u = 0; u < 8; ++u) {
-      l_tot += ws[u] * __shfl(ls, (s0 + u < splits) ? s0 + u : 0, 64);
+      l_tot = range_add(ws[u], __shfl(ls, (s0 + u < splits) ? s0 + u : 0, 64), l_tot);
 #pragma unroll
-      for (int i = 0; i < NF; ++i) acc[i] += ws[u] * ov[u][i];
+      for (int i = 0; i < NF; ++i) acc[i] = range_add(ws[u], ov[u][i], acc[i]);
     }
   }
-  const float inv = 1.0f / l_tot;
 #pragma unroll
   for (int i = 0; i < NF; ++i)
-    if (lane + i * 64 < HD) o[lane + i * 64] = from_float<bf16_t>(acc[i] * inv);
+    if (lane + i * 64 < HD) o[lane + i * 64] = from_float<bf16_t>(range_finish(acc[i], l_tot));
 }
 
 // One wave per (request, head).
@@ -342,7 +341,7 @@ static int launch_decode(bool fused, const DecodeSource& src, void* out, long ou
                          const void* k_cache, const void* v_cache, const int* block_table, int table_width,
                          const int* q_start, const int* kv_len, const int* req_ids, int R, int nh, int nkv, int hd,
                          int page_size, float scale, int window, long num_pages, int splits, void* part, long part_elems,
-                         hipStream_t stream) {
+                         bool merge, hipStream_t stream) {
   PI_REQUIRE(R > 0 && nh > 0 && nkv > 0 && nh % nkv == 0 && nh / nkv <= 16, "attention_decode: needs 1..16 heads per kv head, got %d / %d", nh, nkv);
   PI_REQUIRE(hd >= 16 && hd <= 256 && hd % 16 == 0, "attention_decode: head_dim %d is not a multiple of 16 up to 256", hd);
   PI_REQUIRE(!fused || hd == 64 || hd == 128, "attention_decode: the kernel that starts from the projection takes head_dim 64 or 128, not %d", hd);
@@ -380,7 +379,8 @@ static int launch_decode(bool fused, const DecodeSource& src, void* out, long ou
   }
 #undef GO
   if (pi_check_launch("attention_decode")) return -1;
-  if (splits > 1) return launch_combine(out, out_stride, q_start, req_ids, nullptr, R, part, nh, hd, splits, stream);
+  // merge == false: the caller's next kernel merges the ranges itself (nothing is in `out` then)
+  if (splits > 1 && merge) return launch_combine(out, out_stride, q_start, req_ids, nullptr, R, part, nh, hd, splits, stream);
   return 0;
 }
 
@@ -390,7 +390,7 @@ extern "C" int pi_attention_decode(void* out, long out_stride, const void* q, lo
                                    float scale, int window, long num_pages, int splits, void* part, long part_elems,
                                    hipStream_t stream) {
   return launch_decode(false, DecodeSource{}, out, out_stride, q, q_stride, k_cache, v_cache, block_table, table_width, q_start,
-                       kv_len, req_ids, R, nh, nkv, hd, page_size, scale, window, num_pages, splits, part, part_elems, stream);
+                       kv_len, req_ids, R, nh, nkv, hd, page_size, scale, window, num_pages, splits, part, part_elems, true, stream);
 }
 
 // The same for a step of single tokens only (T == R tokens, request r at row q_start[r]),
@@ -398,12 +398,14 @@ extern "C" int pi_attention_decode(void* out, long out_stride, const void* q, lo
 // [qkv_splits, T, ncols] (one of the two), columns [q heads | k heads | v heads].  `table`:
 // float32 [T, hd] cosines and sines of the tokens' angles (rotation over the whole head, halves
 // paired), or null for no rotation.  write_kv: store the tokens' keys and values into the cache.
+// merge == 0 (with splits > 1): leave the key ranges in `part` ([R, nh, splits, hd + 4]: output
+// not yet normalised, maximum, sum of weights) for a consumer that merges them; `out` stays untouched.
 extern "C" int pi_attention_decode_fused(void* out, long out_stride, const void* qkv, long qkv_stride, const void* qkv_part,
                                          int qkv_splits, int ncols, int T, const float* table, int write_kv, void* k_cache,
                                          void* v_cache, const int* block_table, int table_width, const int* q_start,
                                          const int* kv_len, int R, int nh, int nkv, int hd, int page_size, float scale,
                                          int window, long num_pages, int splits, void* part, long part_elems,
-                                         hipStream_t stream) {
+                                         int merge, hipStream_t stream) {
   PI_REQUIRE((qkv != nullptr) != (qkv_part != nullptr), "attention_decode_fused: give the projection as a tensor or as pieces");
   PI_REQUIRE(T == R, "attention_decode_fused: %d tokens for %d requests (single tokens only)", T, R);
   PI_REQUIRE(nh > 0 && nkv > 0 && hd > 0, "attention_decode_fused: bad sizes");
@@ -431,7 +433,7 @@ extern "C" int pi_attention_decode_fused(void* out, long out_stride, const void*
   src.k_cache = (bf16_t*)k_cache;
   src.v_cache = (bf16_t*)v_cache;
   return launch_decode(true, src, out, out_stride, nullptr, 0, k_cache, v_cache, block_table, table_width, q_start, kv_len,
-                       nullptr, R, nh, nkv, hd, page_size, scale, window, num_pages, splits, part, part_elems, stream);
+                       nullptr, R, nh, nkv, hd, page_size, scale, window, num_pages, splits, part, part_elems, merge != 0, stream);
 }
 
 // Merge partial results that the tile kernel wrote for `Z` tokens whose tiles' keys were cut in

@@ -93,6 +93,21 @@ __device__ inline float split_sum(const float* __restrict__ part, int splits, lo
   return val;
 }
 
+// ---- merging the key ranges of one (token, head): range s brings its un-normalised output,
+// its maximum m (base-2 scale) and its sum of weights l.  One spelling of the arithmetic for
+// every kernel that merges, so that the merged output is the same bits wherever it is made:
+// weights against the overall maximum, sums in range order with fused multiply-adds, one
+// division, one rounding.
+__device__ inline float range_weight(float m, float m_tot) {
+#if defined(__HIP_DEVICE_COMPILE__)
+  return (m == -INFINITY) ? 0.f : __builtin_amdgcn_exp2f(m - m_tot);
+#else
+  return 0.f;
+#endif
+}
+__device__ inline float range_add(float w, float v, float sum) { return __builtin_fmaf(w, v, sum); }
+__device__ inline float range_finish(float acc, float l_tot) { return acc * (1.0f / l_tot); }
+
 // ---- reductions over the four lanes l, l+16, l+32, l+48 (one column of a matrix-core tile),
 // with the gfx950 row / half swaps instead of a trip through the LDS crossbar:
 // v_permlane16_swap exchanges the odd 16-lane rows of one register with the even rows of the

@@ -21,6 +21,7 @@
 enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACCUM = 2, EPI_SWIGLU = 3 };
 
 #define ROWS_PER_BLOCK 32
+#define RANGES_ROW_TILES 4      // row tiles per wave where the key ranges are merged on the way in (fewer blocks repeat the merge)
 #define KSTEP 64
 #define SHARED_FROM_TOKENS 32   // more tokens than this: the kernel that shares an activation tile per block
 #define SHARED_DEPTH 4          // k steps of loads a wave keeps in flight (measured: more is slower)
@@ -36,21 +37,103 @@ __device__ inline void epilogue_store(void* Cv, long ldc, long m, long n, float 
 // memory follow the rows, eight lanes on a row's 128 bytes, which the cache serves at twice the
 // rate of the operand's own pattern of sixteen rows per quarter wave); afterwards the same bytes
 // hold the waves' partial tiles for the sum.
-template <int MB>
+// Activations that are still the key ranges of a decode step's attention (one token per
+// request, request r at row r): float32 [token, head, range, head_dim + 4] holding each range's
+// un-normalised output, then its maximum and its sum of weights.  The product kernel merges
+// them on the way in, which saves the merging kernel between attention and the o projection.
+struct RangeSource {
+  const float* ranges;
+  int heads, head_dim, count;
+};
+
+// Lane group lg merges the key ranges of tokens lg, lg + 4, .. (TOK of them per round) for the
+// lane's four features of one head and leaves them, rounded to bfloat16, where the product's
+// operand reads expect them.  CNT > 0: up to CNT ranges, all loads of a round asked for before
+// the first is used (one trip to memory); CNT == 0: any number, in two passes.  Ranges are added
+// in range order with the shared arithmetic (range_weight / range_add / range_finish).
+template <int CNT, int TOK>
+__device__ inline void merge_ranges_of_tokens(const float* __restrict__ head_base, long token_stride, int count, int rec, int hd,
+                                              int f0, int lg, int lr, int M, uint2* __restrict__ xs2) {
+  const int piece = lr / 2;                              // the 16-byte piece of the k step the lane's features lie in
+#pragma unroll 1
+  for (int t0 = lg; t0 < M; t0 += 4 * TOK) {
+    f32x4_t sum[TOK];
+    float l_tot[TOK];
+    if constexpr (CNT > 0) {
+      float2 ml[TOK][CNT];
+      f32x4_t o[TOK][CNT];
+#pragma unroll
+      for (int j = 0; j < TOK; ++j) {
+        const float* base = head_base + (long)min(t0 + 4 * j, M - 1) * token_stride;
+#pragma unroll
+        for (int u = 0; u < CNT; ++u) {
+          const int r = min(u, count - 1);
+          ml[j][u] = *reinterpret_cast<const float2*>(base + r * rec + hd);
+          o[j][u] = *reinterpret_cast<const f32x4_t*>(base + r * rec + f0);
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < TOK; ++j) {
+        float m_tot = -INFINITY;
+#pragma unroll
+        for (int u = 0; u < CNT; ++u) m_tot = fmaxf(m_tot, ml[j][u].x);
+        sum[j] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        l_tot[j] = 0.f;
+#pragma unroll
+        for (int u = 0; u < CNT; ++u) {
+          const float wgt = u < count ? range_weight(ml[j][u].x, m_tot) : 0.f;
+          l_tot[j] = range_add(wgt, ml[j][u].y, l_tot[j]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e) sum[j][e] = range_add(wgt, o[j][u][e], sum[j][e]);
+        }
+      }
+    } else {
+      static_assert(CNT > 0 || TOK == 1, "the two-pass merge takes one token per round");
+      const float* base = head_base + (long)t0 * token_stride;
+      float m_tot = -INFINITY;
+#pragma unroll 8
+      for (int r = 0; r < count; ++r) m_tot = fmaxf(m_tot, base[r * rec + hd]);
+      sum[0] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+      l_tot[0] = 0.f;
+#pragma unroll 8
+      for (int r = 0; r < count; ++r) {
+        const float2 ml = *reinterpret_cast<const float2*>(base + r * rec + hd);
+        const f32x4_t o = *reinterpret_cast<const f32x4_t*>(base + r * rec + f0);
+        const float wgt = range_weight(ml.x, m_tot);
+        l_tot[0] = range_add(wgt, ml.y, l_tot[0]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sum[0][e] = range_add(wgt, o[e], sum[0][e]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < TOK; ++j) {
+      const int token = t0 + 4 * j;
+      if (token >= M) break;
+      uint2 packed;
+      packed.x = pack_bf16x2(range_finish(sum[j][0], l_tot[j]), range_finish(sum[j][1], l_tot[j]));
+      packed.y = pack_bf16x2(range_finish(sum[j][2], l_tot[j]), range_finish(sum[j][3], l_tot[j]));
+      xs2[(piece * 16 + ((token + 2 * piece) & 15)) * 2 + (lr & 1)] = packed;
+    }
+  }
+}
+
+template <int MB, int RT>
 union SkinnyLds {
-  float red[4][ROWS_PER_BLOCK][MB * 16 + 1];
+  float red[4][RT * 16][MB * 16 + 1];
   u32x4_t xs[4][MB * 8 * 16];          // per wave: [token tile][16-byte piece of the k step][token], tokens turned by the piece
 };
 
-template <int MB, int EPI>
+template <int MB, int EPI, bool RANGES = false, int RT = 2>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ X, long ldx,
                                                           const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
-                                                          int k_per_block, float* __restrict__ part) {
-  __shared__ SkinnyLds<MB> lds;
-  float (*red)[ROWS_PER_BLOCK][MB * 16 + 1] = lds.red;
+                                                          int k_per_block, float* __restrict__ part, RangeSource rs) {
+  constexpr int ROWS = RT * 16;          // weight rows of a block: RT row tiles per wave
+  static_assert(EPI != EPI_SWIGLU || RT == 2, "the SwiGLU epilogue pairs a wave's two row tiles");
+  __shared__ SkinnyLds<MB, RT> lds;
+  float (*red)[ROWS][MB * 16 + 1] = lds.red;
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int lr = lane % 16, lg = lane / 16;
-  const long n0 = (long)blockIdx.x * ROWS_PER_BLOCK;
+  const long n0 = (long)blockIdx.x * ROWS;
   const int splits = gridDim.y;
 
   // this wave's k-range: a quarter (rounded up to whole steps) of the block's range
@@ -61,9 +144,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
   const int k1 = min(kb1, k0 + per_wave);
 
   // rows beyond N read the last valid row; their results are never stored
-  const bf16_t* wrow[2];
+  const bf16_t* wrow[RT];
 #pragma unroll
-  for (int t = 0; t < 2; ++t) wrow[t] = W + min(n0 + t * 16 + lr, (long)N - 1) * ldw + lg * 16;
+  for (int t = 0; t < RT; ++t) wrow[t] = W + min(n0 + t * 16 + lr, (long)N - 1) * ldw + lg * 16;
 
   // Activations of a k step: load instruction i brings tokens 8i .. 8i+7, lane j the 16-byte
   // piece j % 8 of token 8i + j / 8.  Tokens beyond M are not loaded: what LDS holds for them
@@ -85,34 +168,51 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
 #pragma unroll
     for (int h = 0; h < 2; ++h) xfrag[c][h] = (c * 8 + lg * 2 + h) * 16 + ((lr + 2 * (lg * 2 + h)) & 15);
 
-  f32x4_t acc[2][MB];
+  f32x4_t acc[RT][MB];
 #pragma unroll
-  for (int t = 0; t < 2; ++t)
+  for (int t = 0; t < RT; ++t)
 #pragma unroll
     for (int c = 0; c < MB; ++c) acc[t][c] = f32x4_t{0.f, 0.f, 0.f, 0.f};
 
   // one k step; in a last, partial one the 8-element pieces beyond k1 count as zero
   auto step = [&](const int kk, auto whole_step) {
     constexpr bool whole = decltype(whole_step)::value;
-    Frag w[2][2];
+    Frag w[RT][2];
     u32x4_t xg[MB * 2];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < RT; ++t)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
         w[t][h] = load_frag(wrow[t] + (whole || kk + lg * 16 + h * 8 < k1 ? kk + h * 8 : k0));
         if (!whole && kk + lg * 16 + h * 8 >= k1) w[t][h] = zero_frag();
       }
-    const bool x_ok = whole || kk + xp * 8 < k1;
+    if constexpr (RANGES) {
+      // The 64 features of this step belong to one head (head_dim is a multiple of 64).  Lane
+      // group lg merges tokens lg, lg + 4, ..; a lane owns four features.  Every load is asked
+      // for before the first is needed; the ranges are added in range order.
+      static_assert(MB == 1, "merging on the way in serves up to 16 tokens");
+      const int head = kk / rs.head_dim, f0 = kk - head * rs.head_dim + lr * 4;
+      const int rec = rs.head_dim + 4;
+      const float* head_base = rs.ranges + (long)head * rs.count * rec;
+      const long token_stride = (long)rs.heads * rs.count * rec;
+      uint2* xs2 = reinterpret_cast<uint2*>(xs);
+      // tokens per lane group x ranges per token held in registers at once: about 16 either way
+      if (rs.count <= 4) merge_ranges_of_tokens<4, 4>(head_base, token_stride, rs.count, rec, rs.head_dim, f0, lg, lr, M, xs2);
+      else if (rs.count <= 8) merge_ranges_of_tokens<8, 2>(head_base, token_stride, rs.count, rec, rs.head_dim, f0, lg, lr, M, xs2);
+      else if (rs.count <= 16) merge_ranges_of_tokens<16, 1>(head_base, token_stride, rs.count, rec, rs.head_dim, f0, lg, lr, M, xs2);
+      else merge_ranges_of_tokens<0, 1>(head_base, token_stride, rs.count, rec, rs.head_dim, f0, lg, lr, M, xs2);
+    } else {
+      const bool x_ok = whole || kk + xp * 8 < k1;
 #pragma unroll
-    for (int i = 0; i < MB * 2; ++i)
-      if (i == 0 || i < x_loads) {
-        xg[i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + (x_ok ? kk : k0));
-        if (!x_ok) xg[i] = u32x4_t{0u, 0u, 0u, 0u};
-      }
+      for (int i = 0; i < MB * 2; ++i)
+        if (i == 0 || i < x_loads) {
+          xg[i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + (x_ok ? kk : k0));
+          if (!x_ok) xg[i] = u32x4_t{0u, 0u, 0u, 0u};
+        }
 #pragma unroll
-    for (int i = 0; i < MB * 2; ++i)
-      if (i == 0 || i < x_loads) xs[xdst[i]] = xg[i];
+      for (int i = 0; i < MB * 2; ++i)
+        if (i == 0 || i < x_loads) xs[xdst[i]] = xg[i];
+    }
     // the wave reads what its own lanes wrote: LDS serves one wave's accesses in order
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -123,7 +223,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
 #pragma unroll
       for (int h = 0; h < 2; ++h) x[c][h].n = xs[xfrag[c][h]];
 #pragma unroll
-    for (int t = 0; t < 2; ++t)
+    for (int t = 0; t < RT; ++t)
 #pragma unroll
       for (int c = 0; c < MB; ++c) {
         acc[t][c] = mfma16(w[t][0], x[c][0], acc[t][c]);
@@ -139,7 +239,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
 
   // acc[t][c][r] is C^T[n0 + t*16 + lg*4 + r][c*16 + lr]; add the four waves through LDS
 #pragma unroll
-  for (int t = 0; t < 2; ++t)
+  for (int t = 0; t < RT; ++t)
 #pragma unroll
     for (int c = 0; c < MB; ++c)
 #pragma unroll
@@ -158,8 +258,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
         reinterpret_cast<bf16_t*>(Cv)[(long)m * ldc + n0 / 2 + j] = from_float<bf16_t>(g / (1.0f + expf(-g)) * u);
       }
     } else {
-      for (int idx = tid; idx < ROWS_PER_BLOCK * cols; idx += 256) {
-        const int nl = idx % ROWS_PER_BLOCK, m = idx / ROWS_PER_BLOCK;
+      for (int idx = tid; idx < ROWS * cols; idx += 256) {
+        const int nl = idx % ROWS, m = idx / ROWS;
         if (m >= M || n0 + nl >= N) continue;
         epilogue_store<EPI>(Cv, ldc, m, n0 + nl, red[0][nl][m] + red[1][nl][m] + red[2][nl][m] + red[3][nl][m]);
       }
@@ -172,8 +272,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
   // its own read) adds the splits in split order.  No block waits for or signals another:
   // on a chip of several dies a device-wide fence costs more than a kernel boundary.
   float* mine = part + (long)blockIdx.y * M * N;
-  for (int idx = tid; idx < ROWS_PER_BLOCK * cols; idx += 256) {
-    const int nl = idx % ROWS_PER_BLOCK, m = idx / ROWS_PER_BLOCK;
+  for (int idx = tid; idx < ROWS * cols; idx += 256) {
+    const int nl = idx % ROWS, m = idx / ROWS;
     if (m >= M || n0 + nl >= N) continue;
     mine[(long)m * N + n0 + nl] = red[0][nl][m] + red[1][nl][m] + red[2][nl][m] + red[3][nl][m];
   }
@@ -338,7 +438,7 @@ extern "C" int pi_splitk_reduce(void* C, int epilogue, long ldc, const void* par
 template <int MB>
 static int launch_mb(int epi, dim3 grid, hipStream_t stream, void* C, long ldc, const bf16_t* X, long ldx, const bf16_t* W,
                      long ldw, int M, int N, int K, int kpb, float* part) {
-#define GO(E) hipLaunchKernelGGL((gemm_skinny_kernel<MB, E>), grid, dim3(256), 0, stream, C, ldc, X, ldx, W, ldw, M, N, K, kpb, part)
+#define GO(E) hipLaunchKernelGGL((gemm_skinny_kernel<MB, E>), grid, dim3(256), 0, stream, C, ldc, X, ldx, W, ldw, M, N, K, kpb, part, RangeSource{})
   switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
     case EPI_F32: GO(EPI_F32); break;
@@ -401,4 +501,37 @@ extern "C" int pi_gemm_skinny(void* C, int epilogue, long ldc, const void* X, lo
     case 3: return launch_mb<3>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
     default: return launch_mb<4>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
   }
+}
+
+// The same product for a decode step of up to 16 tokens whose activations are attention's key
+// ranges not yet merged (`ranges`: float32 [M, heads, count, head_dim + 4], see RangeSource): K
+// is heads * head_dim, and head_dim a multiple of the kernel's k step so that a step's features
+// belong to one head.  Epilogues: store bf16, store f32, add into f32.
+extern "C" int pi_gemm_skinny_ranges(void* C, int epilogue, long ldc, const void* ranges, int heads, int head_dim, int count,
+                                     const void* W, long ldw, int M, int N, int splits, void* part, long part_elems,
+                                     int* splits_out, hipStream_t stream) {
+  PI_REQUIRE(M > 0 && M <= 16 && N > 0 && heads > 0 && count >= 1 && count <= 64, "gemm_skinny_ranges: takes 1..16 tokens and 1..64 ranges, got M=%d N=%d heads=%d ranges=%d", M, N, heads, count);
+  PI_REQUIRE(head_dim > 0 && head_dim % KSTEP == 0, "gemm_skinny_ranges: head_dim %d is no multiple of %d", head_dim, KSTEP);
+  PI_REQUIRE(epilogue == EPI_BF16 || epilogue == EPI_F32 || epilogue == EPI_ACCUM, "gemm_skinny_ranges: unknown epilogue %d", epilogue);
+  PI_REQUIRE(ldw % 8 == 0 && ((uintptr_t)W % 16 == 0) && ((uintptr_t)ranges % 16 == 0), "gemm_skinny_ranges: operands must be 16-byte aligned");
+  PI_REQUIRE(splits >= 1 && splits <= 65535, "gemm_skinny_ranges: bad split count %d", splits);
+  const long K = (long)heads * head_dim;
+  PI_REQUIRE(K < (1L << 30), "gemm_skinny_ranges: k too long");
+  int kpb = ceil_div((int)K, splits);
+  kpb = ((kpb + 4 * KSTEP - 1) / (4 * KSTEP)) * (4 * KSTEP);     // a block's four waves take whole steps
+  splits = ceil_div((int)K, kpb);
+  if (splits > 1)
+    PI_REQUIRE(part && part_elems >= (long)splits * M * N, "gemm_skinny_ranges: workspace too small (%ld floats for %ld)", part_elems, (long)splits * M * N);
+  if (splits_out) *splits_out = splits;
+  const dim3 grid(ceil_div(N, RANGES_ROW_TILES * 16), splits);
+  const RangeSource rs{(const float*)ranges, heads, head_dim, count};
+#define GO(E) hipLaunchKernelGGL((gemm_skinny_kernel<1, E, true, RANGES_ROW_TILES>), grid, dim3(256), 0, stream, C, ldc, (const bf16_t*)nullptr, 0L, \
+                                 (const bf16_t*)W, ldw, M, N, (int)K, kpb, (float*)part, rs)
+  switch (epilogue) {
+    case EPI_BF16: GO(EPI_BF16); break;
+    case EPI_F32: GO(EPI_F32); break;
+    default: GO(EPI_ACCUM); break;
+  }
+#undef GO
+  return pi_check_launch("gemm_skinny (key ranges merged on the way in)");
 }

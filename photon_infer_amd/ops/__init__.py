@@ -17,7 +17,7 @@ import torch
 
 from ..errors import KernelError
 from . import _lib
-from .workspace import KernelWorkspace, Partials
+from .workspace import KernelWorkspace, KeyRanges, Partials
 
 PI_F32, PI_BF16 = 0, 1
 MAX_HEAD_DIM = 256
@@ -196,6 +196,23 @@ def gemm(out: torch.Tensor, a: torch.Tensor, w: torch.Tensor, accumulate: bool =
     ``may_defer`` (with ``accumulate`` and ``ws``): the caller promises that ``out`` is next read
     by ``rmsnorm`` or ``materialize`` with the same workspace; a product that was split over k may
     then stay in pieces there."""
+    if isinstance(a, KeyRanges):
+        # attention's output of a decode step, its key ranges not merged yet: the weight-streaming
+        # kernel merges them as it reads; anything else gets them merged first
+        _gpu(out, w)
+        if w.dim() != 2 or out.shape != (a.tokens, w.shape[0]) or w.shape[1] != a.heads * a.head_dim:
+            raise KernelError(f"gemm: shapes do not agree: ranges [{a.tokens}, {a.heads} x {a.head_dim}], w {tuple(w.shape)}, out {tuple(out.shape)}")
+        if accumulate:
+            if out.dtype != torch.float32:
+                raise KernelError("gemm: accumulation needs a float32 output")
+            materialize(out, ws)
+        from . import fast
+        if _FAST and fast.gemm_from_ranges(out, a, w, accumulate, w.shape[0], _rows(w, "gemm w"), _rows(out, "gemm out"),
+                                           may_defer and accumulate and out.is_contiguous(), ws):
+            return
+        merged = torch.empty((a.tokens, a.heads * a.head_dim), dtype=torch.bfloat16, device=out.device)
+        fast.merge_ranges(merged, a)
+        a = merged
     _gpu(out, a, w)
     if a.dim() != 2 or w.dim() != 2 or out.dim() != 2:
         raise KernelError("gemm: operands must be 2-D")
@@ -328,12 +345,15 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
 def decode_attention_from_projection(out: torch.Tensor, qkv, ctx, rotary, num_heads: int, num_kv_heads: int,
                                      head_dim: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
                                      block_table: torch.Tensor, page_size: int, scale: float, window: int,
-                                     write_kv: bool, ws: Optional[KernelWorkspace] = None) -> bool:
+                                     write_kv: bool, ws: Optional[KernelWorkspace] = None, leave_ranges: bool = False):
     """For a step that holds single tokens only: rotation, cache write and attention in one
     kernel, from the q|k|v projection ``qkv`` (a tensor [T, N] or ``fast.Partials``, columns
     [q heads | k heads | v heads]).  Returns False, having done nothing, when the step, the
     sizes or the rotation (``rotary`` as for ``rope_kv_write``; only the whole head with paired
-    halves, or none) are not what that kernel serves; the caller then takes the separate kernels."""
+    halves, or none) are not what that kernel serves; the caller then takes the separate kernels.
+    ``leave_ranges`` (needs ``ws``): the caller hands the result straight to ``gemm``; when the
+    keys were split into ranges, the kernel may then return them unmerged (``KeyRanges``, in the
+    workspace) instead of filling ``out``, and the product merges them as it reads."""
     if not (_FAST and out.dtype == torch.bfloat16 and out.is_cuda and getattr(ctx, "all_decode", False)):
         return False
     from . import fast
@@ -353,7 +373,7 @@ def decode_attention_from_projection(out: torch.Tensor, qkv, ctx, rotary, num_he
     if block_table.dim() != 2 or block_table.dtype != torch.int32 or not block_table.is_contiguous():
         raise KernelError("attention: block table must be contiguous int32 [requests, width]")
     return fast.decode_attention_from_projection(out, qkv, ctx, table, num_heads, num_kv_heads, head_dim, k_cache, v_cache,
-                                                 block_table, page_size, scale, window, pages, write_kv, ws)
+                                                 block_table, page_size, scale, window, pages, write_kv, ws, leave_ranges)
 
 
 def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,

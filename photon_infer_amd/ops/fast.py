@@ -23,7 +23,7 @@ import numpy as np
 import torch
 
 from . import _lib
-from .workspace import GEMM_PART_FLOATS, KernelWorkspace, Partials, PendingUpdate
+from .workspace import GEMM_PART_FLOATS, KernelWorkspace, KeyRanges, Partials, PendingUpdate
 
 EPI_BF16, EPI_F32, EPI_ACCUM, EPI_SWIGLU = 0, 1, 2, 3
 SKINNY_MAX_ROWS = 128          # up to this many tokens the weight-streaming kernels serve a product (measured against the tile kernel)
@@ -161,6 +161,55 @@ def gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc, may_defer=False, ws: Opt
         else:
             _lib.call("bf16", "pi_splitk_reduce", out.data_ptr(), epilogue, ldc, pieces.part.data_ptr(), pieces.splits,
                       M, N, _stream())
+    return True
+
+
+RANGES_MAX_TOKENS = 16      # the weight-streaming kernel merges key ranges on the way in for up to this many tokens
+RANGES_HEAD_DIM_STEP = 64   # ... of heads whose size is a multiple of its k step
+
+
+def ranges_product_ok(tokens: int, head_dim: int) -> bool:
+    return tokens <= RANGES_MAX_TOKENS and head_dim % RANGES_HEAD_DIM_STEP == 0
+
+
+def merge_ranges(out: torch.Tensor, kr: KeyRanges) -> None:
+    """The merged attention output, bfloat16 [tokens, heads * head_dim], by the merging kernel."""
+    _lib.call("bf16", "pi_attention_combine_rows", out.data_ptr(), out.stride(0), kr.rows.data_ptr(), kr.tokens,
+              kr.part.data_ptr(), kr.heads, kr.head_dim, kr.count, _stream())
+
+
+def gemm_from_ranges(out, kr: KeyRanges, w, accumulate, N, ldw, ldc, may_defer, ws: Optional[KernelWorkspace]) -> bool:
+    """out (+)= merged(kr) @ w^T by the weight-streaming kernel, which merges the key ranges as it
+    stages its activations; the same bits as merging first."""
+    M, K = kr.tokens, kr.heads * kr.head_dim
+    if not ranges_product_ok(M, kr.head_dim) or w.dtype != torch.bfloat16 or w.stride(1) != 1 or ldw % 8 or w.data_ptr() % 16:
+        return False
+    if accumulate:
+        epilogue = EPI_ACCUM
+    elif out.dtype == torch.bfloat16:
+        epilogue = EPI_BF16
+    elif out.dtype == torch.float32:
+        epilogue = EPI_F32
+    else:
+        return False
+    splits = _skinny_splits(M, N, K)
+    buf = _piece_buffer(ws, splits * M * N, w.device) if splits > 1 else None
+    made = ctypes.c_int(0)
+    _lib.call("bf16", "pi_gemm_skinny_ranges", out.data_ptr(), epilogue, ldc, kr.part.data_ptr(), kr.heads, kr.head_dim, kr.count,
+              w.data_ptr(), ldw, M, N, splits, None if buf is None else buf.data_ptr(), 0 if buf is None else buf.numel(),
+              ctypes.byref(made), _stream())
+    if ws is not None:
+        ws.counts["ranges_merged_by_product"] += 1
+    if made.value > 1:
+        pieces = Partials(buf, made.value, M, N)
+        if ws is not None:
+            ws.counts["split_products"] += 1
+        if may_defer and ws is not None:
+            ws.pending = PendingUpdate(out, pieces)
+            ws.counts["deferred"] += 1
+        else:
+            _lib.call("bf16", "pi_splitk_reduce", out.data_ptr(), epilogue, ldc, pieces.part.data_ptr(), pieces.splits, M, N,
+                      _stream())
     return True
 
 
@@ -432,10 +481,12 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
 
 def decode_attention_from_projection(out, qkv, ctx, table, num_heads, num_kv_heads, head_dim, k_cache, v_cache,
                                      block_table, page_size, scale, window, pages, write_kv,
-                                     ws: Optional[KernelWorkspace] = None) -> bool:
+                                     ws: Optional[KernelWorkspace] = None, leave_ranges: bool = False):
     """A step of single tokens: attention straight from the q|k|v projection (``qkv``: a bfloat16
     tensor [T, N] or ``Partials``), which the kernel rotates by ``table`` (the step's cos / sin
-    table [T, head_dim], or None) and whose keys and values it stores.  False: not for these sizes."""
+    table [T, head_dim], or None) and whose keys and values it stores.  False: not for these sizes.
+    ``leave_ranges``: when the keys were split into ranges and the product that reads the output
+    can merge them (``ranges_product_ok``), they are returned as ``KeyRanges`` and ``out`` is left alone."""
     G = num_heads // num_kv_heads
     if not ctx.all_decode or G > 16 or head_dim not in FUSED_DECODE_HEAD_DIMS or page_size % 16 or out.stride(0) % 4:
         return False
@@ -448,11 +499,14 @@ def decode_attention_from_projection(out, qkv, ctx, table, num_heads, num_kv_hea
         return False
     splits = _decode_splits_that_fit(ws, R, num_heads, num_kv_heads, head_dim, ctx.max_kv_len)
     part = _attn_part(ws, R * num_heads * splits * (head_dim + 4), out.device)
+    leave = leave_ranges and ws is not None and splits > 1 and ranges_product_ok(R, head_dim)
     _lib.call("bf16", "pi_attention_decode_fused", out.data_ptr(), out.stride(0),
               None if pieces else qkv.data_ptr(), 0 if pieces else qkv.stride(0),
               qkv.part.data_ptr() if pieces else None, qkv.splits if pieces else 0, qkv.N if pieces else 0, R,
               None if table is None else table.data_ptr(), int(bool(write_kv)), k_cache.data_ptr(), v_cache.data_ptr(),
               block_table.data_ptr(), block_table.shape[1], ctx.q_start.data_ptr(), ctx.kv_len.data_ptr(), R, num_heads,
               num_kv_heads, head_dim, page_size, float(scale), int(window), pages, splits, part.data_ptr(),
-              part.numel(), _stream())
+              part.numel(), int(not leave), _stream())
+    if leave:
+        return KeyRanges(part, splits, R, num_heads, head_dim, ctx.q_start)
     return True

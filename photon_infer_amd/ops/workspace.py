@@ -31,6 +31,25 @@ class Partials:
 
 
 @dataclass
+class KeyRanges:
+    """The attention output of a decode step (token r is request r) whose key ranges are not
+    merged yet: ``part`` holds float32 [tokens, heads, count, head_dim + 4] (a range's output not
+    yet normalised, then its maximum and its sum of weights).  It lives in the workspace's
+    attention buffer, so it has to be consumed (``ops.gemm`` takes it as its activations) before
+    the next attention of that workspace runs.  ``rows``: int32 device array, row of each token."""
+
+    part: torch.Tensor
+    count: int
+    tokens: int
+    heads: int
+    head_dim: int
+    rows: torch.Tensor
+
+    def __bool__(self) -> bool:
+        return True
+
+
+@dataclass
 class PendingUpdate:
     """``target += sum(pieces)`` that has not been applied yet."""
 
@@ -45,7 +64,7 @@ class PendingUpdate:
 class KernelWorkspace:
     """Buffers are made at first use and kept; ``counts`` says which paths a step took (tests
     read it: ``split_products``, ``deferred``, ``added_by_norm``, ``applied``, ``flushed``,
-    ``discarded``, ``qkv_pieces``)."""
+    ``discarded``, ``qkv_pieces``, ``ranges_merged_by_product``)."""
 
     def __init__(self, device):
         self.device = torch.device(device)

@@ -102,10 +102,12 @@ class PagedAttention(Mixer):
         if qkv is not None and ctx.all_decode:
             # single tokens only: one kernel rotates, writes the cache and attends
             attn = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
-            if ops.decode_attention_from_projection(attn, qkv, ctx, rotary, self.num_heads, self.num_kv_heads,
-                                                    self.head_dim, cache.k, cache.v, table, cache.page_size, self.scale,
-                                                    self.window or 0, writes, ws):
-                ops.gemm(x, attn, self.w_o, accumulate=True, may_defer=True, ws=ws)
+            done = ops.decode_attention_from_projection(attn, qkv, ctx, rotary, self.num_heads, self.num_kv_heads,
+                                                        self.head_dim, cache.k, cache.v, table, cache.page_size, self.scale,
+                                                        self.window or 0, writes, ws, leave_ranges=True)
+            if done:
+                # the output, or its key ranges still to be merged, which the product does as it reads them
+                ops.gemm(x, done if isinstance(done, ops.KeyRanges) else attn, self.w_o, accumulate=True, may_defer=True, ws=ws)
                 return
         if qkv is not None and not isinstance(qkv, torch.Tensor):
             # the projection is still in pieces (split over k): the rotation kernel sums them

@@ -469,6 +469,35 @@ def test_decode_attention_from_projection(_ops, hd, nh, nkv, page, window, rotat
     k3 = k2.clone()
     assert _ops.decode_attention_from_projection(got2, qkv, ctx, rotary, nh, nkv, hd, k3, v2, kv.table, page, scale, window, False)
     assert torch.equal(got2, apart) and torch.equal(k3, k2)
+    # the key ranges left unmerged for the product that reads the output next: the o projection
+    # merges them as it stages its activations, to the same bits as the merging kernel
+    ws = _ops.KernelWorkspace(DEV)
+    k4, v4 = kv.k.clone(), kv.v.clone()
+    untouched = torch.full((R, nh * hd), 7.0, dtype=BF16, device=DEV)
+    ranges = _ops.decode_attention_from_projection(untouched, qkv, ctx, rotary, nh, nkv, hd, k4, v4, kv.table, page, scale, window,
+                                                   True, ws, leave_ranges=True)
+    assert isinstance(ranges, _ops.KeyRanges) and ranges.count > 1 and torch.equal(k4, k1) and torch.equal(v4, v1)
+    assert (untouched == 7.0).all()
+    for n_out, w_dtype in ((96, BF16), (40, BF16), (200, F32)):
+        w_o = (torch.randn(n_out, nh * hd, generator=g) * 0.05).to(w_dtype).to(DEV)
+        x0 = torch.randn(R, n_out, generator=g).to(DEV)
+        want_x, got_x = x0.clone(), x0.clone()
+        _ops.gemm(want_x, apart, w_o, accumulate=True)
+        _ops.gemm(got_x, ranges, w_o, accumulate=True, ws=ws)
+        assert torch.equal(got_x, want_x), f"o projection from key ranges, {n_out} x {w_dtype}"
+        want_b, got_b = torch.empty(R, n_out, dtype=BF16, device=DEV), torch.empty(R, n_out, dtype=BF16, device=DEV)
+        _ops.gemm(want_b, apart, w_o)
+        _ops.gemm(got_b, ranges, w_o, ws=ws)
+        assert torch.equal(got_b, want_b)
+    assert ws.counts["ranges_merged_by_product"] == 4              # the float32 weights went through the merging kernel
+    # and left in pieces for the stream's next norm, as the model's o projection is
+    w_o = (torch.randn(96, nh * hd, generator=g) * 0.05).to(BF16).to(DEV)
+    x0 = torch.randn(R, 96, generator=g).to(DEV)
+    want_x, got_x = x0.clone(), x0.clone()
+    _ops.gemm(want_x, apart, w_o, accumulate=True)
+    _ops.gemm(got_x, ranges, w_o, accumulate=True, may_defer=True, ws=ws)
+    _ops.materialize(got_x, ws)
+    assert torch.equal(got_x, want_x)
 
 
 def test_decode_attention_from_projection_declines_what_it_does_not_serve(_ops):

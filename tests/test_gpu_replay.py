@@ -66,11 +66,13 @@ LENGTHS = {"A": [5, 9, 17, 70, 128], "B": [1, 7, 33, 64, 100, 200], "C": [3, 48,
            "F": [1, 140, 300], "G": [2, 50, 270]}
 
 
-def check_kernel_selection(runner, name, dtype, portions=True, single_tokens=True):
+def check_kernel_selection(runner, name, dtype, decoded_alone=False):
     """Model F is there so that the kernels chosen at real sizes run inside these comparisons: in
     bfloat16 its o and down projections are split over k and left in pieces that the next norm
     adds, and its q|k|v projection reaches the rotation (portions) or the fused decode kernel
-    (single tokens) in pieces.  The workspace counts say whether a run went that way."""
+    (single tokens) in pieces; where steps of single tokens alone ran late in a sequence
+    (``decoded_alone``), attention left its key ranges for the o projection to merge.  The
+    workspace counts say whether a run went that way."""
     counts = runner.workspace.counts
     if name != "F" or dtype != "bfloat16":
         if dtype == "float32":
@@ -79,6 +81,8 @@ def check_kernel_selection(runner, name, dtype, portions=True, single_tokens=Tru
     assert counts["split_products"] > 0 and counts["deferred"] > 0 and counts["qkv_pieces"] > 0, counts
     assert counts["added_by_norm"] == counts["deferred"] - counts["flushed"] - counts["applied"] - counts["discarded"], counts
     assert counts["flushed"] == 0, counts               # every pending update found its norm
+    if decoded_alone:
+        assert counts["ranges_merged_by_product"] > 0, counts
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -104,7 +108,7 @@ def test_last_32_tokens_one_by_one(model_dirs, tmp_path, name, dtype):
     steps = cut_steps("r0", toks, [n - 32] + [1] * 32)
     runner = runner_for(model_dirs[name], name, dtype, live_token_need(steps))
     check(run_trace(runner, steps, str(tmp_path)), model_dirs[name], reqs, dtype, "tail decoded")
-    check_kernel_selection(runner, name, dtype)
+    check_kernel_selection(runner, name, dtype, decoded_alone=True)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
