@@ -8,19 +8,20 @@
 // of them from the pages into registers while all four compute on the previous 128, which
 // they share through LDS (stored in the very order the matrix-core operands want them, so
 // both the writes and the reads are 16 bytes per lane, lane after lane).  One barrier per 128
-// keys.  A token at absolute position p sees keys lo..p only (lo = 0, or p - window + 1),
+// keys.  Heads of more than 128 features take 64 keys at a time (two of the waves fetch) and
+// 16 columns per wave: two rounds of 128 would not fit the LDS, nor the state the registers.  A token at absolute position p sees keys lo..p only (lo = 0, or p - window + 1),
 // whatever portion it arrived in; a wave skips the 32-key chunks none of its columns sees.
 //
 // The host sorts the tiles by the number of keys they walk and deals them out to the blocks
 // of a kv head in rounds, back and forth, so that every block gets about the same work.
 #include "attention_mfma.h"
 
-#define KEYS_PER_ROUND 128
 #ifndef PLAIN_NJ
 #define PLAIN_NJ 4   // chunks of a fully visible round that are folded as one group (2 or 4)
 #endif
 
-template <int HD, int CB>
+// NCH: chunks of 32 keys per round (4, or 2 for the large heads)
+template <int HD, int CB, int NCH>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 2 : 1))) void attention_tiles_kernel(
     bf16_t* __restrict__ out, long out_stride, const bf16_t* __restrict__ q, long q_stride,
     const bf16_t* __restrict__ k_cache, const bf16_t* __restrict__ v_cache, const int* __restrict__ block_table,
@@ -30,7 +31,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
     int nkv, int page_size, float scale, int window, long num_pages_l, int TQ) {
   constexpr int KS = HeadFrags<HD>::KS;
   constexpr int F = 2 * KS + HD / 16;             // 16-byte operand fragments per lane and 32 keys: keys, then values
-  extern __shared__ __attribute__((aligned(16))) u32x4_t staged[];   // [2 buffers][4 chunks][F][64 lanes]
+  constexpr int KEYS_PER_ROUND = NCH * 32;
+  static_assert(NCH == 2 || NCH == 4, "a round is two or four chunks");
+  extern __shared__ __attribute__((aligned(16))) u32x4_t staged[];   // [2 buffers][NCH chunks][F][64 lanes]
   __shared__ int present[2][4][2];                // is the page of a 16-key tile there
   const int lane = threadIdx.x % 64;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64);
@@ -90,11 +93,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
       attn_load_q(st, c, q, q_stride, rows[c], heads[c], valid[c], lane);
     }
 
-    // this wave's 32 keys of every 128: where they lie
+    // this wave's 32 keys of every round (the first NCH waves fetch): where they lie
+    const bool fetches = wave < NCH;
     PageCursor cur;
     cur.start(block_table + (long)r * table_width, table_width, kv_len, page_size, sc0 * KEYS_PER_ROUND + wave * 32);
     KVChunk<HD> pre;
     auto fetch = [&]() {
+      if (!fetches) return;
       PageCursor two = cur;                        // the chunk's two tiles
       const ChunkPages cp = two.next();
       attn_load<HD>(pre, cp, k_cache, v_cache, off, nkv, g, page_size, num_pages);
@@ -104,7 +109,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
       if (cur.slot >= page_size) { cur.slot -= page_size; ++cur.blk; }
     };
     auto stash = [&](int buf) {
-      u32x4_t* mine = staged + ((buf * 4 + wave) * F) * 64 + lane;
+      if (!fetches) return;
+      u32x4_t* mine = staged + ((buf * NCH + wave) * F) * 64 + lane;
 #pragma unroll
       for (int t = 0; t < 2; ++t)
 #pragma unroll
@@ -124,17 +130,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
       // a round that every column of the wave sees whole, with every page there: straight-line
       // code without the per-key tests (the accumulators then stay in place from chunk to chunk)
       const int round0 = sc * KEYS_PER_ROUND;
-      const bool missing = __builtin_amdgcn_ballot_w64(lane < 8 && !(&present[buf][0][0])[lane % 8]) != 0;
+      const bool missing = __builtin_amdgcn_ballot_w64(lane < 2 * NCH && !(&present[buf][0][0])[lane % 8]) != 0;
+      constexpr int NJ = NCH < PLAIN_NJ ? NCH : PLAIN_NJ;
       if (active && !missing && round0 >= see_all_lo && round0 + KEYS_PER_ROUND - 1 <= see_all_hi) {
-        attn_compute_plain<HD, CB, PLAIN_NJ>(st, staged + (buf * 4 * F) * 64 + lane, F * 64, scale_log2);
-        if (PLAIN_NJ < 4) attn_compute_plain<HD, CB, PLAIN_NJ>(st, staged + ((buf * 4 + 2) * F) * 64 + lane, F * 64, scale_log2);
+        attn_compute_plain<HD, CB, NJ>(st, staged + (buf * NCH * F) * 64 + lane, F * 64, scale_log2);
+        if (NJ < NCH) attn_compute_plain<HD, CB, NJ>(st, staged + ((buf * NCH + 2) * F) * 64 + lane, F * 64, scale_log2);
       } else if (active) {
 #pragma unroll 1
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < NCH; ++j) {
           const int key0 = sc * KEYS_PER_ROUND + j * 32;
           if (key0 > see_any_hi || key0 + 31 < see_any_lo) continue;
           StagedChunk<HD> kv;
-          kv.from = staged + ((buf * 4 + j) * F) * 64 + lane;
+          kv.from = staged + ((buf * NCH + j) * F) * 64 + lane;
           kv.have[0] = __builtin_amdgcn_readfirstlane(present[buf][j][0]) != 0;
           kv.have[1] = __builtin_amdgcn_readfirstlane(present[buf][j][1]) != 0;
           const bool masked = key0 < see_all_lo || key0 + 31 > see_all_hi || !kv.have[0] || !kv.have[1];
@@ -183,12 +190,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
 // Tokens per tile for a head layout: the block's columns divided among the heads of a group.
 extern "C" int pi_attention_tile_rows(int nh, int nkv, int hd) {
   if (nkv <= 0 || nh <= 0 || nh % nkv) return 0;
-  const int cols = 4 * 2 * 16;
+  const int cols = 4 * (hd > 128 ? 1 : 2) * 16;   // four waves of two column blocks, one for the large heads
   return cols / (nh / nkv);
 }
 
-// Shared memory of one block: two buffers of 128 keys and their values.
-static size_t tiles_lds_bytes(int hd) { return (size_t)2 * 4 * (2 * ((hd + 31) / 32) + hd / 16) * 64 * 16; }
+// Shared memory of one block: two buffers of a round's keys and values (128 keys, or 64 for the large heads).
+static size_t tiles_lds_bytes(int hd) { return (size_t)2 * (hd > 128 ? 2 : 4) * (2 * ((hd + 31) / 32) + hd / 16) * 64 * 16; }
 
 // `order`: [rounds, seats] tile indices (-1: none), the host's deal of the tiles to `seats`
 // blocks per kv head.  tile_cut[t] = cut | cuts << 8: which of how many shares of its keys entry
@@ -201,7 +208,7 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
                                          int nkv, int hd, int page_size, float scale, int window, long num_pages,
                                          hipStream_t stream) {
   PI_REQUIRE(rounds > 0 && seats > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_prefill: bad sizes rounds=%d seats=%d heads=%d kv_heads=%d", rounds, seats, nh, nkv);
-  PI_REQUIRE(hd >= 16 && hd <= 128 && hd % 16 == 0, "attention_prefill: head_dim %d is not a multiple of 16 up to 128", hd);
+  PI_REQUIRE(hd >= 16 && hd <= 256 && hd % 16 == 0, "attention_prefill: head_dim %d is not a multiple of 16 up to 256", hd);
   PI_REQUIRE(page_size >= 16 && page_size % 16 == 0, "attention_prefill: page size %d must be a multiple of 16", page_size);
   PI_REQUIRE(table_width >= 1, "attention_prefill: empty block table");
   const int TQ = pi_attention_tile_rows(nh, nkv, hd);
@@ -210,28 +217,36 @@ extern "C" int pi_attention_prefill_mfma(void* out, long out_stride, const void*
   PI_REQUIRE(out_stride % 4 == 0 && q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && ((uintptr_t)out % 8 == 0), "attention_prefill: q / out rows must be 16- / 8-byte aligned");
   const size_t lds = tiles_lds_bytes(hd);
   const dim3 grid(nkv, seats), block(256);
-#define GO(H, C)                                                                                                                           \
+#define GO(H, C, N)                                                                                                                          \
   do {                                                                                                                                     \
     static bool configured = false;                                                                                                        \
     if (!configured) {                                                                                                                     \
-      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_tiles_kernel<H, C>),                                      \
+      hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(attention_tiles_kernel<H, C, N>),                                      \
                                          hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);                                            \
       if (e != hipSuccess) return pi_fail("attention_prefill: cannot reserve %zu bytes of LDS: %s", lds, hipGetErrorString(e));            \
       configured = true;                                                                                                                   \
     }                                                                                                                                      \
-    hipLaunchKernelGGL((attention_tiles_kernel<H, C>), grid, block, lds, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride,     \
+    hipLaunchKernelGGL((attention_tiles_kernel<H, C, N>), grid, block, lds, stream, (bf16_t*)out, out_stride, (const bf16_t*)q, q_stride,     \
                        (const bf16_t*)k_cache, (const bf16_t*)v_cache, block_table, table_width, q_start, kv_len, tile_req, tile_q0,       \
                        tile_cut, tile_z0, (float*)part, order, rounds, nh, nkv, page_size, scale, window, num_pages, TQ);                  \
   } while (0)
   switch (hd) {
-    case 16: GO(16, 2); break;
-    case 32: GO(32, 2); break;
-    case 48: GO(48, 2); break;
-    case 64: GO(64, 2); break;
-    case 80: GO(80, 2); break;
-    case 96: GO(96, 2); break;
-    case 112: GO(112, 2); break;
-    default: GO(128, 2); break;
+    case 16: GO(16, 2, 4); break;
+    case 32: GO(32, 2, 4); break;
+    case 48: GO(48, 2, 4); break;
+    case 64: GO(64, 2, 4); break;
+    case 80: GO(80, 2, 4); break;
+    case 96: GO(96, 2, 4); break;
+    case 112: GO(112, 2, 4); break;
+    case 128: GO(128, 2, 4); break;
+    case 144: GO(144, 1, 2); break;
+    case 160: GO(160, 1, 2); break;
+    case 176: GO(176, 1, 2); break;
+    case 192: GO(192, 1, 2); break;
+    case 208: GO(208, 1, 2); break;
+    case 224: GO(224, 1, 2); break;
+    case 240: GO(240, 1, 2); break;
+    default: GO(256, 1, 2); break;
   }
 #undef GO
   return pi_check_launch("attention_prefill_mfma");

@@ -10,7 +10,7 @@ Which kernel takes what:
   * attention: pages of a multiple of 16 tokens; a batch of single tokens with at most 16 heads
     per kv head goes to the key-split decode kernel (head_dim a multiple of 16 up to 256; for
     64 and 128 straight from the q|k|v projection), any other batch to the tile kernel
-    (head_dim a multiple of 16 up to 128), its single tokens to the decode kernel.
+    (head_dim a multiple of 16 up to 256), its single tokens to the decode kernel.
 """
 from __future__ import annotations
 
@@ -36,7 +36,7 @@ TILE_MAX_SPLITS = 4
 BIG_MIN_TILES = 192            # 256 x 256 tiles (times k pieces) from which the large-tile kernel is taken (the library's rule)
 BIG_MIN_K = 1024               # a piece of the large-tile kernel keeps at least this much of k
 PIECES_BELOW_TILES = 200       # fewer 128 x 128 tiles than this: q, k, v of a prompt portion are left in k pieces too
-TILE_HEAD_DIMS = tuple(range(16, 129, 16))         # head sizes of the prompt-attention tile kernel (its LDS holds two rounds of keys and values)
+TILE_HEAD_DIMS = tuple(range(16, 257, 16))         # head sizes of the prompt-attention tile kernel (above 128: rounds of 64 keys, 16 columns per wave)
 DECODE_HEAD_DIMS = tuple(range(16, 257, 16))       # head sizes of the key-split decode kernel
 FUSED_DECODE_HEAD_DIMS = (64, 128)                 # ... and of its form that starts from the q|k|v projection (whole halves of a head per fragment)
 MAX_DECODE_SPLITS = 64         # the combine kernel holds one key range per lane

@@ -547,8 +547,8 @@ ATTN_CASES = [
     (8, 2, 64, 64, [130, 3, 1], [130, 250, 99], 33),                 # portions with a window, pages of 64
     (16, 1, 64, 16, [1, 1], [129, 2], None),                         # sixteen heads on one kv head
     (32, 1, 64, 16, [1, 70], [75, 70], None),                        # more heads per kv head than a wave's columns
-    # the other head sizes of the matrix-core kernels: every multiple of 16 up to 128 (tile and decode
-    # kernel) and up to 256 (decode kernel); sizes that are no multiple of 32 end in half a fragment
+    # the other head sizes of the matrix-core kernels: every multiple of 16 up to 256; sizes that are
+    # no multiple of 32 end in half a fragment
     (4, 2, 16, 16, [1, 20, 1], [40, 20, 300], None),
     (3, 1, 48, 16, [33, 1, 2], [33, 90, 130], None),
     (4, 4, 80, 16, [1, 5, 1], [90, 37, 600], 16),
@@ -565,7 +565,16 @@ ATTN_CASES = [
     (4, 1, 192, 16, [1, 1], [50, 700], None),
     (8, 2, 224, 16, [1], [300], 100),
     (2, 2, 256, 16, [1, 1, 1], [1, 33, 400], None),
-    (4, 1, 192, 16, [5, 1], [50, 700], None),                        # a portion at a head size the tile kernel does not take
+    # portions at head sizes above 128: the tile kernel in rounds of 64 keys, 16 columns per wave
+    (4, 1, 192, 16, [5, 1], [50, 700], None),
+    (2, 2, 144, 16, [70, 1, 3], [300, 20, 64], None),
+    (6, 2, 160, 32, [40, 1, 2, 100], [40, 77, 300, 100], None),
+    (3, 1, 176, 16, [33, 17], [33, 90], 48),
+    (4, 4, 208, 16, [65, 2], [200, 130], None),
+    (8, 2, 224, 16, [20, 1], [150, 300], 100),
+    (2, 1, 240, 16, [64], [64], None),
+    (8, 2, 256, 16, [130, 3, 1], [130, 250, 99], 33),
+    (4, 1, 256, 16, [37, 1], [2600, 900], None),                     # few tiles, many keys: cut and merged at head size 256
     (8, 2, 128, 16, [1, 70, 1, 1, 2], [900, 300, 33, 1, 50], None),  # single tokens beside portions: two kernels share the step
     (4, 2, 64, 16, [1, 3, 1], [700, 40, 18], 25),                    # the same with a window
     (8, 2, 64, 16, [70, 5], [2100, 40], None),                       # few tiles, many keys: their key ranges are cut and merged

@@ -19,7 +19,7 @@ pytestmark = pytest.mark.gpu
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DTYPES = ["float32", "bfloat16"]
-MODELS = ["A", "B", "C", "D", "E", "F", "G"]
+MODELS = ["A", "B", "C", "D", "E", "F", "G", "H"]
 
 _plain_cache = {}
 
@@ -63,7 +63,7 @@ def check(got, model_dir, reqs, dtype, what):
 
 
 LENGTHS = {"A": [5, 9, 17, 70, 128], "B": [1, 7, 33, 64, 100, 200], "C": [3, 48, 131], "D": [1, 31, 65, 300], "E": [2, 33, 129, 260],
-           "F": [1, 140, 300], "G": [2, 50, 270]}
+           "F": [1, 140, 300], "G": [2, 50, 270], "H": [3, 70, 260]}
 
 
 def check_kernel_selection(runner, name, dtype, decoded_alone=False):
@@ -102,7 +102,7 @@ def test_each_request_alone_and_whole(model_dirs, tmp_path, name, dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", MODELS)
 def test_last_32_tokens_one_by_one(model_dirs, tmp_path, name, dtype):
-    n = {"A": 100, "B": 180, "C": 150, "D": 260, "E": 200, "F": 290, "G": 190}[name]
+    n = {"A": 100, "B": 180, "C": 150, "D": 260, "E": 200, "F": 290, "G": 190, "H": 210}[name]
     reqs = requests_for(name, [n], seed=1)
     toks = reqs["r0"]
     steps = cut_steps("r0", toks, [n - 32] + [1] * 32)
@@ -114,7 +114,7 @@ def test_last_32_tokens_one_by_one(model_dirs, tmp_path, name, dtype):
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("name", MODELS)
 def test_portions_of_changing_size(model_dirs, tmp_path, name, dtype):
-    n = {"A": 120, "B": 230, "C": 170, "D": 290, "E": 210, "F": 280, "G": 200}[name]
+    n = {"A": 120, "B": 230, "C": 170, "D": 290, "E": 210, "F": 280, "G": 200, "H": 220}[name]
     reqs = requests_for(name, [n], seed=2)
     # F also in portions that the tile kernels take (more than 128 tokens), split over k
     for sizes in ([7, 2, 16, 3, 2, 33, 1, 5], [2], [64, 2, 2, 19]) + (([130, 2, 140],) if name == "F" else ()):
@@ -162,7 +162,7 @@ def test_mixed_requests_with_pages_used_again(model_dirs, tmp_path, name, dtype)
     lengths = {"A": [40, 9, 128, 77, 5, 100, 64, 30], "B": [100, 1, 33, 250, 64, 7, 180, 90],
                "C": [131, 48, 3, 200, 96, 150], "D": [300, 65, 2, 129, 500, 17, 210],
                "E": [260, 33, 2, 129, 400, 64, 97], "F": [300, 65, 2, 129, 260, 17, 210],
-               "G": [200, 33, 2, 129, 300, 64, 80]}[name]
+               "G": [200, 33, 2, 129, 300, 64, 80], "H": [180, 33, 2, 129, 290, 64, 70]}[name]
     reqs = requests_for(name, lengths, seed=3)
     pats = [[16, 1, 1, 1, 2], [1], [33, 2, 7], [64, 1, 1], [5, 3, 2], [2, 2, 50], [1, 1, 1, 40], [9]]
     patterns = {rid: pats[i % len(pats)] for i, rid in enumerate(reqs)}

@@ -82,9 +82,18 @@ TINY_G = dict(
 )
 TINY_G_INIT = dict(std=0.07, norm_init="uniform", block_size=16)
 
+# H: a head of 160 features, above what two rounds of 128 keys allow in the LDS: prompts go
+# through the tile kernel in rounds of 64 keys with 16 columns per wave; two heads on one kv head
+TINY_H = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=112, intermediate_size=200, num_hidden_layers=2,
+    num_attention_heads=2, num_key_value_heads=1, head_dim=160, vocab_size=410, max_position_embeddings=512,
+    rms_norm_eps=1e-6, rope_theta=10000.0, tie_word_embeddings=False,
+)
+TINY_H_INIT = dict(std=0.06, norm_init="uniform", block_size=16)
+
 ALL = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT), "D": (TINY_D, TINY_D_INIT),
        "E": (TINY_E, TINY_E_INIT), "F": (TINY_F, TINY_F_INIT),
-       "G": (TINY_G, TINY_G_INIT)}
+       "G": (TINY_G, TINY_G_INIT), "H": (TINY_H, TINY_H_INIT)}
 
 
 def make_model_dir(tmp_path, name: str, seed: int = 0, storage: str = "bfloat16") -> str:
