@@ -345,15 +345,16 @@ def rope_kv_write(q: torch.Tensor, k: Optional[torch.Tensor], v: Optional[torch.
 def decode_attention_from_projection(out: torch.Tensor, qkv, ctx, rotary, num_heads: int, num_kv_heads: int,
                                      head_dim: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
                                      block_table: torch.Tensor, page_size: int, scale: float, window: int,
-                                     write_kv: bool, ws: Optional[KernelWorkspace] = None, leave_ranges: bool = False):
+                                     write_kv: bool, ws: Optional[KernelWorkspace] = None, leave_ranges: int = 0):
     """For a step that holds single tokens only: rotation, cache write and attention in one
     kernel, from the q|k|v projection ``qkv`` (a tensor [T, N] or ``fast.Partials``, columns
     [q heads | k heads | v heads]).  Returns False, having done nothing, when the step, the
     sizes or the rotation (``rotary`` as for ``rope_kv_write``; only the whole head with paired
     halves, or none) are not what that kernel serves; the caller then takes the separate kernels.
-    ``leave_ranges`` (needs ``ws``): the caller hands the result straight to ``gemm``; when the
-    keys were split into ranges, the kernel may then return them unmerged (``KeyRanges``, in the
-    workspace) instead of filling ``out``, and the product merges them as it reads."""
+    ``leave_ranges`` (needs ``ws``; 0, or the bytes of the weight matrix the result goes to): the
+    caller hands the result straight to ``gemm`` with that matrix; when the keys were split into
+    ranges, the kernel may then return them unmerged (``KeyRanges``, in the workspace) instead of
+    filling ``out``, and the product merges them as it reads."""
     if not (_FAST and out.dtype == torch.bfloat16 and out.is_cuda and getattr(ctx, "all_decode", False)):
         return False
     from . import fast

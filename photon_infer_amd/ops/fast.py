@@ -166,10 +166,14 @@ def gemm(out, a, w, accumulate, M, N, K, lda, ldw, ldc, may_defer=False, ws: Opt
 
 RANGES_MAX_TOKENS = 16      # the weight-streaming kernel merges key ranges on the way in for up to this many tokens
 RANGES_HEAD_DIM_STEP = 64   # ... of heads whose size is a multiple of its k step
+# ... and for weights up to this size: the merging kernel has 64 weight rows per block, half the
+# blocks of the plain one, which a larger matrix needs to stream at full rate (measured, batch 1
+# to 16 at context 4,096: 8.4 MB 1 to 3 % faster per step, 19 MB and 34 MB 2 to 6 % slower)
+RANGES_MAX_WEIGHT_BYTES = 12 << 20
 
 
-def ranges_product_ok(tokens: int, head_dim: int) -> bool:
-    return tokens <= RANGES_MAX_TOKENS and head_dim % RANGES_HEAD_DIM_STEP == 0
+def ranges_product_ok(tokens: int, head_dim: int, weight_bytes: int = 0) -> bool:
+    return tokens <= RANGES_MAX_TOKENS and head_dim % RANGES_HEAD_DIM_STEP == 0 and weight_bytes <= RANGES_MAX_WEIGHT_BYTES
 
 
 def merge_ranges(out: torch.Tensor, kr: KeyRanges) -> None:
@@ -182,7 +186,7 @@ def gemm_from_ranges(out, kr: KeyRanges, w, accumulate, N, ldw, ldc, may_defer, 
     """out (+)= merged(kr) @ w^T by the weight-streaming kernel, which merges the key ranges as it
     stages its activations; the same bits as merging first."""
     M, K = kr.tokens, kr.heads * kr.head_dim
-    if not ranges_product_ok(M, kr.head_dim) or w.dtype != torch.bfloat16 or w.stride(1) != 1 or ldw % 8 or w.data_ptr() % 16:
+    if not ranges_product_ok(M, kr.head_dim, N * K * 2) or w.dtype != torch.bfloat16 or w.stride(1) != 1 or ldw % 8 or w.data_ptr() % 16:
         return False
     if accumulate:
         epilogue = EPI_ACCUM
@@ -254,7 +258,12 @@ def attention_tile_rows(num_heads: int, num_kv_heads: int, head_dim: int) -> int
     return _lib.load("bf16").pi_attention_tile_rows(num_heads, num_kv_heads, head_dim)
 
 
-ATTENTION_BLOCKS_PER_UNIT = 2   # blocks of the tile kernel that fit one compute unit (LDS, registers)
+def attention_blocks_per_unit(head_dim: int) -> int:
+    """Blocks of the tile kernel that one compute unit holds at a time: two up to head size 64,
+    one above (its LDS and registers).  More seats than that only queue behind the first and
+    leave the deal of tiles to blocks uneven: at head size 128 a 2,048-token prompt took 104 us
+    with two seats per unit and 84 us with one."""
+    return 2 if head_dim <= 64 else 1
 
 
 def deal_tiles(walks: List[int], seats: int) -> np.ndarray:
@@ -282,6 +291,7 @@ class AttentionPlanner:
     num_kv_heads: int
     singles_apart: bool       # requests that bring one token go to the key-split kernel instead
     units: int                # compute units of the device
+    blocks_per_unit: int = 2  # blocks that a unit holds at a time (attention_blocks_per_unit)
 
     def plan(self, q_lens: Sequence[int], kv_lens: Sequence[int]):
         """None for a step of single tokens only (the key-split kernel needs no list); otherwise
@@ -307,7 +317,7 @@ class AttentionPlanner:
                     first_row.append(row0 + start)
                     n_tok.append(min(tile_rows, n - start))
             row0 += n
-        seats_wanted = max(1, ATTENTION_BLOCKS_PER_UNIT * self.units // max(1, self.num_kv_heads))
+        seats_wanted = max(1, self.blocks_per_unit * self.units // max(1, self.num_kv_heads))
         # too few tiles for the chip (a portion of a few hundred tokens): cut the key range of
         # the long ones into equal shares; the shares' partial results are merged afterwards
         cuts = cut_count(walks, seats_wanted)
@@ -346,7 +356,8 @@ def attention_planner(dtype, num_heads: int, num_kv_heads: int, head_dim: int, p
     if tile_rows < 1:
         return None
     units = torch.cuda.get_device_properties(device).multi_processor_count
-    return AttentionPlanner(tile_rows, int(window), num_kv_heads, num_heads // num_kv_heads <= 16, units)
+    return AttentionPlanner(tile_rows, int(window), num_kv_heads, num_heads // num_kv_heads <= 16, units,
+                            attention_blocks_per_unit(head_dim))
 
 
 def upload_arrays(arrays: Dict[str, np.ndarray], device) -> Dict[str, torch.Tensor]:
@@ -397,17 +408,26 @@ class TilePlan:
 
 
 MAX_TILE_CUTS = 8
+MIN_ROUNDS_PER_SHARE = 4       # a share of a cut tile walks at least this many rounds of 128 keys ...
+MIN_ROUNDS_SAVED = 6           # ... and the cut shortens the longest walk by at least this many
 
 
 def cut_count(walks: List[int], seats_wanted: int) -> int:
     """In how many shares the key range of a step's long tiles is cut: 1 unless the tiles are
-    fewer than half the blocks the chip holds; then as many as fill it, while every share keeps
-    at least two rounds of 128 keys."""
+    fewer than half the blocks the chip holds; then as many as fill it, while a share keeps
+    enough rounds of 128 keys to be worth an entry of its own (its queries loaded again, its
+    partial result written and merged: about the time of six rounds).  Measured at head sizes
+    64 and 128, 64 to 1,024 tokens ending at 256 to 8,192: shares of two rounds made 256 tokens
+    at 2,048 slower than uncut (56 us against 46; with shares of four 29 us), and two shares of
+    a walk of eight rounds or less never paid."""
     tiles = len(walks)
     if tiles == 0 or tiles * 2 > seats_wanted:
         return 1
-    cuts = min(MAX_TILE_CUTS, seats_wanted // tiles, max(walks) // 2)
-    return max(1, cuts)
+    longest = max(walks)
+    cuts = min(MAX_TILE_CUTS, seats_wanted // tiles, longest // MIN_ROUNDS_PER_SHARE)
+    if cuts < 2 or longest - -(-longest // cuts) < MIN_ROUNDS_SAVED:
+        return 1
+    return cuts
 
 
 def decode_length_bucket(max_kv_len: int) -> int:
@@ -481,12 +501,13 @@ def paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_k
 
 def decode_attention_from_projection(out, qkv, ctx, table, num_heads, num_kv_heads, head_dim, k_cache, v_cache,
                                      block_table, page_size, scale, window, pages, write_kv,
-                                     ws: Optional[KernelWorkspace] = None, leave_ranges: bool = False):
+                                     ws: Optional[KernelWorkspace] = None, leave_ranges: int = 0):
     """A step of single tokens: attention straight from the q|k|v projection (``qkv``: a bfloat16
     tensor [T, N] or ``Partials``), which the kernel rotates by ``table`` (the step's cos / sin
     table [T, head_dim], or None) and whose keys and values it stores.  False: not for these sizes.
-    ``leave_ranges``: when the keys were split into ranges and the product that reads the output
-    can merge them (``ranges_product_ok``), they are returned as ``KeyRanges`` and ``out`` is left alone."""
+    ``leave_ranges`` (0: never; else the bytes of the weight matrix that reads the output next):
+    when the keys were split into ranges and that product can merge them (``ranges_product_ok``),
+    they are returned as ``KeyRanges`` and ``out`` is left alone."""
     G = num_heads // num_kv_heads
     if not ctx.all_decode or G > 16 or head_dim not in FUSED_DECODE_HEAD_DIMS or page_size % 16 or out.stride(0) % 4:
         return False
@@ -499,7 +520,7 @@ def decode_attention_from_projection(out, qkv, ctx, table, num_heads, num_kv_hea
         return False
     splits = _decode_splits_that_fit(ws, R, num_heads, num_kv_heads, head_dim, ctx.max_kv_len)
     part = _attn_part(ws, R * num_heads * splits * (head_dim + 4), out.device)
-    leave = leave_ranges and ws is not None and splits > 1 and ranges_product_ok(R, head_dim)
+    leave = leave_ranges > 0 and ws is not None and splits > 1 and ranges_product_ok(R, head_dim, leave_ranges)
     _lib.call("bf16", "pi_attention_decode_fused", out.data_ptr(), out.stride(0),
               None if pieces else qkv.data_ptr(), 0 if pieces else qkv.stride(0),
               qkv.part.data_ptr() if pieces else None, qkv.splits if pieces else 0, qkv.N if pieces else 0, R,

@@ -104,7 +104,8 @@ class PagedAttention(Mixer):
             attn = torch.empty((T, self.q_size), dtype=self.dtype, device=h.device)
             done = ops.decode_attention_from_projection(attn, qkv, ctx, rotary, self.num_heads, self.num_kv_heads,
                                                         self.head_dim, cache.k, cache.v, table, cache.page_size, self.scale,
-                                                        self.window or 0, writes, ws, leave_ranges=True)
+                                                        self.window or 0, writes, ws,
+                                                        leave_ranges=self.w_o.numel() * self.w_o.element_size())
             if done:
                 # the output, or its key ranges still to be merged, which the product does as it reads them
                 ops.gemm(x, done if isinstance(done, ops.KeyRanges) else attn, self.w_o, accumulate=True, may_defer=True, ws=ws)

@@ -204,8 +204,8 @@ def test_late_portions_of_a_long_prompt(model_dirs, tmp_path, dtype, monkeypatch
     """Short portions near the end of the longest context the model allows, beside a second
     request's single tokens: in bfloat16 the portions' few tiles have their key ranges cut
     into shares, and the single tokens go to the key-split kernel in the same step."""
-    reqs = requests_for("D", [500, 130], seed=6)
-    a = cut_steps("r0", reqs["r0"], [440, 40, 3, 17])
+    reqs = requests_for("D", [1500, 130], seed=6)
+    a = cut_steps("r0", reqs["r0"], [1440, 40, 3, 17])
     b = cut_steps("r1", reqs["r1"], [127, 1, 1, 1])
     steps = [b[0], a[0]]
     for i in range(1, 4):                                   # steps that hold a late portion of r0 and one token of r1

@@ -49,7 +49,10 @@ def test_key_ranges_of_tiles_are_cut_only_when_the_tiles_are_few():
     assert cut_count([20] * 64, 64) == 1 and cut_count([20] * 33, 64) == 1      # enough tiles: none is cut
     assert cut_count([64] * 16, 64) == 4                                        # 16 tiles, 64 blocks wanted
     assert cut_count([64] * 2, 64) == MAX_TILE_CUTS
-    assert cut_count([5] * 16, 64) == 2                                         # a share keeps two rounds at least
+    assert cut_count([5] * 16, 64) == 1 and cut_count([7] * 2, 64) == 1         # a share keeps four rounds at least
+    assert cut_count([12] * 4, 64) == 3
+    assert cut_count([8] * 8, 64) == 1 and cut_count([9] * 16, 64) == 1         # ... and the cut saves six rounds or it is not made
+    assert cut_count([16] * 16, 64) == 4
     assert cut_count([1] * 4, 64) == 1
 
 

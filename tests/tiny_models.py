@@ -40,7 +40,7 @@ TINY_C_INIT = dict(std=0.12, norm_init="uniform", block_size=16)
 # that the bfloat16 engine runs them: 2 heads per kv head, llama3 scaling with a short context
 TINY_D = dict(
     architectures=["LlamaForCausalLM"], hidden_size=128, intermediate_size=272, num_hidden_layers=2,
-    num_attention_heads=4, num_key_value_heads=2, head_dim=64, vocab_size=520, max_position_embeddings=512,
+    num_attention_heads=4, num_key_value_heads=2, head_dim=64, vocab_size=520, max_position_embeddings=2048,
     rms_norm_eps=1e-5, rope_theta=50000.0,
     rope_scaling=dict(rope_type="llama3", factor=4.0, low_freq_factor=1.0, high_freq_factor=4.0,
                       original_max_position_embeddings=128),
