@@ -94,7 +94,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(HD <= 64 ? 
     }
 
     // this wave's 32 keys of every round (the first NCH waves fetch): where they lie
-    const bool fetches = wave < NCH;
+    // (a constant where every wave fetches: behind a branch the compiler waits for the loads at
+    // the branch's end instead of at their first use, and the round loses its overlap: 63 us
+    // instead of 53 for a 2,048-token prompt at head size 64)
+    const bool fetches = NCH == 4 || wave < NCH;
     PageCursor cur;
     cur.start(block_table + (long)r * table_width, table_width, kv_len, page_size, sc0 * KEYS_PER_ROUND + wave * 32);
     KVChunk<HD> pre;

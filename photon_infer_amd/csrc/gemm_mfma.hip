@@ -1,8 +1,14 @@
 // bfloat16 matrix product on the matrix cores for many rows (prompts):
 //   C[M, N] (+)= A[M, K] . W[N, K]^T, float32 accumulation.
 // Block tile 128 x 128, reduction slab 64, four waves in 2 x 2, each wave 64 x 64 as 2 x 2
-// tiles of v_mfma_f32_32x32x16_bf16.  Slabs go global -> registers -> LDS (double buffered,
-// rows padded to 144 bytes so 16-byte fragment reads do not collide on banks).
+// tiles of v_mfma_f32_32x32x16_bf16.  Slabs go from memory straight into LDS (buffer loads
+// with the LDS as their destination, double buffered): no registers and no LDS store
+// instructions in between.  Such a load writes its 64 lanes' 16 bytes one after the other, so
+// rows cannot be padded; instead the 16-byte pieces of a row are turned by (row / 2) % 8, which
+// puts the fragment reads of sixteen neighbouring rows on all 64 banks.  (Through registers
+// and padded rows, which this kernel did first, the q/k/v product of a 2,048-token prompt took
+// 40 us instead of 34 and the 256 x 256 kernel below 133 us instead of 120 on the gate / up
+// product: 230 instead of 180 registers, eight LDS stores per slab and thread.)
 //
 // Epilogues: store bfloat16, store float32, add into float32 (the residual stream), or
 // SwiGLU: with gate and up rows interleaved in blocks of 16 in W, the gate and the up value of
@@ -21,8 +27,7 @@ PI_DEFINE_MODULE(bf16)
 #define BM 128
 #define BN 128
 #define BK 64
-#define LDS_ROW (BK + 8)                    // bf16 elements per padded row
-#define TILE_ELEMS (BM * LDS_ROW)
+#define TILE_ELEMS (BM * BK)                // a tile's slab in LDS: rows of 128 bytes
 
 enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACCUM = 2, EPI_SWIGLU = 3 };
 
@@ -139,8 +144,10 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
                                                         const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
                                                         int tiles_n, int k_per_split) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-  uint16_t* As = lds;                       // [2][BM][LDS_ROW]
-  uint16_t* Ws = lds + 2 * TILE_ELEMS;      // [2][BN][LDS_ROW]
+  constexpr int ROW = BK;                   // rows of 128 bytes, no padding (see the large-tile kernel)
+  constexpr int TILE = BM * ROW;
+  uint16_t* As = lds;                       // [2][BM][ROW], 16-byte pieces of a row turned by (row / 2) % 8
+  uint16_t* Ws = lds + 2 * TILE;            // [2][BN][ROW]
   const int tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
   const int wm = wave / 2, wn = wave % 2;
   // k split over blocks (gridDim.y > 1, float32 store only): split s owns k in
@@ -163,43 +170,39 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
   }
   const long m0 = (long)tile_m * BM, n0 = (long)tile_n * BN;
 
-  // global -> register staging: thread t moves 16-byte chunk (t % 8) of rows (t / 8) + 32 p
-  // (eight lanes move one row's 128 bytes; the next eight lanes take the row 8 further down, so
-  // that sixteen lanes land on 64 distinct LDS banks with rows 144 bytes apart)
-  const int lgrp = tid / 8, lchunk = tid % 8;
-  const int lrow = (lgrp / 16) * 16 + ((lgrp / 8) % 2) * 4 + (lgrp % 8) / 2 + 8 * (lgrp % 2);
+  // global -> LDS without registers in between: load instruction p of wave w fills rows
+  // (4 w + p) * 8 .. + 7 of a tile, lane l the 16-byte piece l % 8 of row l / 8, which is piece
+  // (l % 8) ^ ((row / 2) % 8) of the row in memory.  Rows beyond the matrix and k beyond the
+  // range take an offset outside the descriptor and arrive as zeros.
   const int a_rows = (int)min((long)BM, M - m0), w_rows = (int)min((long)BN, N - n0);
 #if defined(__HIP_DEVICE_COMPILE__)
   const __amdgpu_buffer_rsrc_t a_src = operand_descriptor(A + m0 * lda + k_lo, ((long)(a_rows - 1) * lda + (k_hi - k_lo)) * 2);
   const __amdgpu_buffer_rsrc_t w_src = operand_descriptor(W + n0 * ldw + k_lo, ((long)(w_rows - 1) * ldw + (k_hi - k_lo)) * 2);
 #endif
   unsigned a_off[4], w_off[4];
+  int piece_k[4];                           // first k (inside a slab) of the piece this lane fetches
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
-    const int row = lrow + 32 * p;
-    a_off[p] = row < a_rows ? (unsigned)(row * (int)lda + lchunk * 8) * 2u : PI_OUT_OF_RANGE;
-    w_off[p] = row < w_rows ? (unsigned)(row * (int)ldw + lchunk * 8) * 2u : PI_OUT_OF_RANGE;
+    const int row = (wave * 4 + p) * 8 + lane / 8;
+    const int piece = (lane % 8) ^ ((row >> 1) & 7);
+    piece_k[p] = piece * 8;
+    a_off[p] = row < a_rows ? (unsigned)(row * (int)lda + piece * 8) * 2u : PI_OUT_OF_RANGE;
+    w_off[p] = row < w_rows ? (unsigned)(row * (int)ldw + piece * 8) * 2u : PI_OUT_OF_RANGE;
   }
-  u32x4_t ra[4], rw[4];
-  auto load_slab = [&](int k0) {
-    // k0 is relative to k_lo; this lane's 8 k of the slab may lie beyond the range (last slab)
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  auto load_slab = [&](int k0, int buf) {
+    // k0 is relative to k_lo; a lane's 8 k of the slab may lie beyond the range (last slab)
     const unsigned kb = (unsigned)k0 * 2u;
-    const bool k_in = k0 + lchunk * 8 < k_hi - k_lo;
 #if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
-      ra[p] = __builtin_amdgcn_raw_buffer_load_b128(a_src, k_in ? a_off[p] + kb : PI_OUT_OF_RANGE, 0, 0);
-      rw[p] = __builtin_amdgcn_raw_buffer_load_b128(w_src, k_in ? w_off[p] + kb : PI_OUT_OF_RANGE, 0, 0);
+      const bool k_in = k0 + piece_k[p] < k_hi - k_lo;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_src, (lds_ptr_t)(As + buf * TILE + (wave * 4 + p) * 8 * ROW), 16,
+                                               k_in ? a_off[p] + kb : PI_OUT_OF_RANGE, 0, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(w_src, (lds_ptr_t)(Ws + buf * TILE + (wave * 4 + p) * 8 * ROW), 16,
+                                               k_in ? w_off[p] + kb : PI_OUT_OF_RANGE, 0, 0, 0);
     }
 #endif
-  };
-  auto store_slab = [&](int buf) {
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      const int off = (lrow + 32 * p) * LDS_ROW + lchunk * 8;
-      *reinterpret_cast<u32x4_t*>(As + buf * TILE_ELEMS + off) = ra[p];
-      *reinterpret_cast<u32x4_t*>(Ws + buf * TILE_ELEMS + off) = rw[p];
-    }
   };
 
   f32x16_t acc[2][2];
@@ -211,17 +214,20 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
   const int slabs = (k_hi - k_lo + BK - 1) / BK;
-  // 32 x 32 x 16 instruction: a lane reads row lane % 32, 16 bytes at k = (lane / 32) * 8; with
-  // rows 144 bytes apart the 16 lanes served together fall on distinct banks
-  const int frow = lane % 32, fk = (lane / 32) * 8;
+  // 32 x 32 x 16 instruction: a lane reads row lane % 32, the 16 bytes of k = (lane / 32) * 8 of
+  // every 16 k, at the place its row's turn puts them
+  const int frow = lane % 32;
+  int place[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) place[ks] = ((ks * 2 + lane / 32) ^ ((frow >> 1) & 7)) * 8;
   Frag fa[2][2], fb[2][2];
   auto read_frags = [&](int which, int buf, int ks) {   // ks: which 16 k of the slab
-    const uint16_t* a_base = As + buf * TILE_ELEMS + (wm * 64 + frow) * LDS_ROW + fk + ks * 16;
-    const uint16_t* w_base = Ws + buf * TILE_ELEMS + (wn * 64 + frow) * LDS_ROW + fk + ks * 16;
+    const uint16_t* a_base = As + buf * TILE + (wm * 64 + frow) * ROW + place[ks];
+    const uint16_t* w_base = Ws + buf * TILE + (wn * 64 + frow) * ROW + place[ks];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) fa[which][i].n = *reinterpret_cast<const u32x4_t*>(a_base + i * 32 * LDS_ROW);
+    for (int i = 0; i < 2; ++i) fa[which][i].n = *reinterpret_cast<const u32x4_t*>(a_base + i * 32 * ROW);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) fb[which][j].n = *reinterpret_cast<const u32x4_t*>(w_base + j * 32 * LDS_ROW);
+    for (int j = 0; j < 2; ++j) fb[which][j].n = *reinterpret_cast<const u32x4_t*>(w_base + j * 32 * ROW);
   };
   auto products = [&](int which) {
 #pragma unroll
@@ -233,6 +239,9 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
   // descriptor's range) into the buffer nobody reads.  Fragments of the next 16 k are read
   // while the matrix instructions of these 16 run; the hints deal one memory instruction of
   // each kind named after every matrix instruction.
+  // The loop has no branch: a slab beyond the range arrives as zeros in the buffer nobody reads.
+  // Fragments of the next 16 k are read while the matrix instructions of these 16 run; the hints
+  // deal one memory instruction of each kind named after every matrix instruction.
 #define PI_SCHED_MFMA 0x008
 #define PI_SCHED_VMEM_READ 0x020
 #define PI_SCHED_DS_READ 0x100
@@ -243,28 +252,27 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
     if (kind_a) __builtin_amdgcn_sched_group_barrier(kind_a, 1, 0);                  \
     if (kind_b) __builtin_amdgcn_sched_group_barrier(kind_b, 2, 0);                  \
   }
-  load_slab(0);
-  store_slab(0);
+  load_slab(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0): this wave's pieces of the slab are in LDS
   __syncthreads();
-  load_slab(BK);
   read_frags(0, 0, 0);
   for (int s = 0; s < slabs; ++s) {
     const int buf = s & 1;
+    load_slab((s + 1) * BK, buf ^ 1);       // into the buffer everybody left at the last barrier; beyond the range: zeros, unused
     read_frags(1, buf, 1);
     products(0);
-    PI_DEAL4(PI_SCHED_DS_READ, 0)
+    PI_DEAL4(PI_SCHED_DS_READ, PI_SCHED_VMEM_READ)
     read_frags(0, buf, 2);
     products(1);
     PI_DEAL4(PI_SCHED_DS_READ, 0)
     read_frags(1, buf, 3);
     products(0);
-    store_slab(buf ^ 1);            // slab s + 1, loaded while slab s - 1's last step ran
-    PI_DEAL4(PI_SCHED_DS_READ, PI_SCHED_DS_WRITE)
+    PI_DEAL4(PI_SCHED_DS_READ, 0)
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    load_slab((s + 2) * BK);
     read_frags(0, buf ^ 1, 0);
     products(1);
-    PI_DEAL4(PI_SCHED_DS_READ, PI_SCHED_VMEM_READ)
+    PI_DEAL4(PI_SCHED_DS_READ, 0)
   }
 #undef PI_DEAL4
   __syncthreads();                  // the fragments read last belong to no slab; LDS is free for the patches
@@ -285,28 +293,30 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
 
 // ---------------------------------------------------------------------------------------------
 // The same product with block tile 256 x 256 for problems that have enough of them to fill the
-// chip and a k that is a multiple of the slab: four waves in 2 x 2, each 128 x 128 as 4 x 4
-// tiles of v_mfma_f32_32x32x16_bf16.  Per 16 k a wave reads 8 fragments from LDS for 16
-// matrix-core instructions, half the LDS traffic per flop of the 128 x 128 kernel.  The
-// accumulators alone are 256 registers, so there is one wave per SIMD and nothing else to fill
-// its idle cycles: every load, LDS access and address computation has to be issued in the
-// shadow of a matrix-core instruction (32 cycles each).  Hence no branch in the loop (rows
-// beyond the matrix are clamped on load and skipped on store), global loads through a buffer
-// descriptor (a scalar base that moves with k plus fixed 32-bit lane offsets, no vector
-// arithmetic per slab), and scheduling hints that deal the memory instructions out between
-// the matrix-core ones.  A slab's global loads are issued a whole slab before they are stored.
+// chip and a k that is a multiple of the slab: eight waves in 2 x 4 (two per SIMD), each
+// 128 x 64 as 4 x 2 tiles of v_mfma_f32_32x32x16_bf16.  Per 16 k a wave reads 6 fragments from
+// LDS for 8 matrix-core instructions, three quarters of the LDS traffic per flop of the
+// 128 x 128 kernel, and a block asks L2 for half the bytes per flop.  With one wave per SIMD
+// (four waves of 128 x 128, the first form of this kernel) every barrier and every wait left
+// the matrix pipe idle.  No branch in the loop (rows beyond the matrix are clamped on load and
+// skipped on store), loads through a buffer descriptor (a scalar base that moves with k plus
+// fixed 32-bit lane offsets, no vector arithmetic per slab) straight into the other LDS
+// buffer, issued at the top of a slab and awaited at its one barrier, and scheduling hints that
+// deal the memory instructions out between the matrix-core ones.
 // Per output element the sum over k runs in ascending k, as in the small kernel.
 #define GM 256
 #define GN 256
-#define BIG_TILE_ELEMS (GM * LDS_ROW)
+#define BIG_TILE_ELEMS (GM * BK)
 
 template <int EPI>
 __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ A, long lda,
                                                             const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
                                                             int tiles_n, int k_per_split) {
   extern __shared__ __attribute__((aligned(16))) uint16_t lds[];
-  uint16_t* As = lds;                           // [2][GM][LDS_ROW]
-  uint16_t* Ws = lds + 2 * BIG_TILE_ELEMS;      // [2][GN][LDS_ROW]
+  constexpr int ROW = BK;                       // rows of 128 bytes, no padding: the loads write LDS themselves, lane after lane
+  constexpr int TILE = GM * ROW;
+  uint16_t* As = lds;                           // [2][GM][ROW], 16-byte pieces of a row turned by (row / 2) % 8
+  uint16_t* Ws = lds + 2 * TILE;                // [2][GN][ROW]
   const int tid = threadIdx.x, lane = tid % 64;
   const int wave = __builtin_amdgcn_readfirstlane(tid / 64);
   const int wm = wave / 4, wn = wave % 4;       // a wave's corner: 128 rows x 64 columns
@@ -325,9 +335,10 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
   }
   const long m0 = (long)tile_m * GM, n0 = (long)tile_n * GN;
 
-  // global -> registers: thread t moves 16-byte chunk t % 8 of rows lrow + 64 p of both operands
-  const int lgrp = tid / 8, lchunk = tid % 8;
-  const int lrow = (lgrp / 16) * 16 + ((lgrp / 8) % 2) * 4 + (lgrp % 8) / 2 + 8 * (lgrp % 2);
+  // global -> LDS without registers in between: load instruction p of wave w fills rows
+  // (4 w + p) * 8 .. + 7 of a tile, lane l the 16-byte piece l % 8 of row l / 8.  Which piece of
+  // the row in memory that is depends on the row: piece c of row r lies at place c ^ ((r / 2) % 8),
+  // so that the fragment reads of sixteen neighbouring rows fall on all 64 banks.
   const int a_rows = (int)min((long)GM, M - m0), w_rows = (int)min((long)GN, N - n0);
 #if defined(__HIP_DEVICE_COMPILE__)
   const __amdgpu_buffer_rsrc_t a_src = operand_descriptor(A + m0 * lda + k_lo, ((long)(a_rows - 1) * lda + (k_hi - k_lo)) * 2);
@@ -336,28 +347,22 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
   unsigned a_off[4], w_off[4];
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
-    a_off[p] = (unsigned)(min(lrow + 64 * p, a_rows - 1) * (int)lda + lchunk * 8) * 2u;
-    w_off[p] = (unsigned)(min(lrow + 64 * p, w_rows - 1) * (int)ldw + lchunk * 8) * 2u;
+    const int row = (wave * 4 + p) * 8 + lane / 8;
+    const int piece = (lane % 8) ^ ((row >> 1) & 7);
+    a_off[p] = (unsigned)(min(row, a_rows - 1) * (int)lda + piece * 8) * 2u;
+    w_off[p] = (unsigned)(min(row, w_rows - 1) * (int)ldw + piece * 8) * 2u;
   }
-  u32x4_t ra[4], rw[4];
   const int slabs = (k_hi - k_lo) / BK;
-  auto load_slab = [&](int s) {
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  auto load_slab = [&](int s, int buf) {
     const int kbytes = min(s, slabs - 1) * BK * 2;     // past the last slab: read it again, unused
 #if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
-      ra[p] = __builtin_amdgcn_raw_buffer_load_b128(a_src, a_off[p], kbytes, 0);
-      rw[p] = __builtin_amdgcn_raw_buffer_load_b128(w_src, w_off[p], kbytes, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(a_src, (lds_ptr_t)(As + buf * TILE + (wave * 4 + p) * 8 * ROW), 16, a_off[p], kbytes, 0, 0);
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(w_src, (lds_ptr_t)(Ws + buf * TILE + (wave * 4 + p) * 8 * ROW), 16, w_off[p], kbytes, 0, 0);
     }
 #endif
-  };
-  auto store_slab = [&](int buf) {
-#pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      const int off = (lrow + 64 * p) * LDS_ROW + lchunk * 8;
-      *reinterpret_cast<u32x4_t*>(As + buf * BIG_TILE_ELEMS + off) = ra[p];
-      *reinterpret_cast<u32x4_t*>(Ws + buf * BIG_TILE_ELEMS + off) = rw[p];
-    }
   };
 
   f32x16_t acc[4][2];
@@ -368,15 +373,18 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
 #pragma unroll
       for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
 
-  const int frow = lane % 32, fk = (lane / 32) * 8;
+  const int frow = lane % 32;
+  int place[4];                                  // where this lane's piece of each 16 k lies in its rows
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) place[ks] = ((ks * 2 + lane / 32) ^ ((frow >> 1) & 7)) * 8;
   Frag fa[2][4], fb[2][2];
   auto read_frags = [&](int which, int buf, int ks) {   // ks: which 16 k of the slab
-    const uint16_t* a_base = As + buf * BIG_TILE_ELEMS + (wm * 128 + frow) * LDS_ROW + fk + ks * 16;
-    const uint16_t* w_base = Ws + buf * BIG_TILE_ELEMS + (wn * 64 + frow) * LDS_ROW + fk + ks * 16;
+    const uint16_t* a_base = As + buf * TILE + (wm * 128 + frow) * ROW + place[ks];
+    const uint16_t* w_base = Ws + buf * TILE + (wn * 64 + frow) * ROW + place[ks];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) fa[which][i].n = *reinterpret_cast<const u32x4_t*>(a_base + i * 32 * LDS_ROW);
+    for (int i = 0; i < 4; ++i) fa[which][i].n = *reinterpret_cast<const u32x4_t*>(a_base + i * 32 * ROW);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) fb[which][j].n = *reinterpret_cast<const u32x4_t*>(w_base + j * 32 * LDS_ROW);
+    for (int j = 0; j < 2; ++j) fb[which][j].n = *reinterpret_cast<const u32x4_t*>(w_base + j * 32 * ROW);
   };
   auto products = [&](int which) {
 #pragma unroll
@@ -385,10 +393,9 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
       for (int j = 0; j < 2; ++j) acc[i][j] = mfma32(fa[which][i], fb[which][j], acc[i][j]);
   };
 
-  load_slab(0);
-  store_slab(0);
+  load_slab(0, 0);
+  __builtin_amdgcn_s_waitcnt(0x0F70);           // vmcnt(0): this wave's pieces of the slab are in LDS
   __syncthreads();
-  load_slab(1);
   read_frags(0, 0, 0);
   // the order wanted inside one scheduling region: one matrix-core instruction, then one of
   // each kind of memory instruction named, `n` times; the rest of the 8 after that
@@ -400,25 +407,25 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
   }
   for (int s = 0; s < slabs; ++s) {
     const int buf = s & 1;
+    load_slab(s + 1, buf ^ 1);      // into the buffer everybody left at the last barrier
     read_frags(1, buf, 1);
     products(0);
-    PI_DEAL(6, PI_SCHED_DS_READ, 0)
-    PI_DEAL(2, 0, 0)
+    PI_DEAL(6, PI_SCHED_DS_READ, PI_SCHED_VMEM_READ)
+    PI_DEAL(2, PI_SCHED_VMEM_READ, 0)
     read_frags(0, buf, 2);
     products(1);
     PI_DEAL(6, PI_SCHED_DS_READ, 0)
     PI_DEAL(2, 0, 0)
     read_frags(1, buf, 3);
     products(0);
-    store_slab(buf ^ 1);            // slab s + 1, loaded during the previous slab's last step
-    PI_DEAL(6, PI_SCHED_DS_READ, PI_SCHED_DS_WRITE)
-    PI_DEAL(2, PI_SCHED_DS_WRITE, 0)
+    PI_DEAL(6, PI_SCHED_DS_READ, 0)
+    PI_DEAL(2, 0, 0)
+    __builtin_amdgcn_s_waitcnt(0x0F70);
     __syncthreads();
-    load_slab(s + 2);
     read_frags(0, buf ^ 1, 0);
     products(1);
-    PI_DEAL(6, PI_SCHED_VMEM_READ, PI_SCHED_DS_READ)
-    PI_DEAL(2, PI_SCHED_VMEM_READ, 0)
+    PI_DEAL(6, PI_SCHED_DS_READ, 0)
+    PI_DEAL(2, 0, 0)
   }
 #undef PI_DEAL
 
@@ -437,10 +444,10 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
   }
 }
 
-static const size_t kBigLdsBytes = 4 * BIG_TILE_ELEMS * sizeof(uint16_t);   // 147,456 bytes
+static const size_t kBigLdsBytes = 4 * BIG_TILE_ELEMS * sizeof(uint16_t);   // 131,072 bytes
 #define BIG_MIN_TILES 192      // enough 256 x 256 tiles (times k pieces) to occupy most of the chip
 
-static const size_t kLdsBytes = 4 * TILE_ELEMS * sizeof(uint16_t);   // 73,728 bytes
+static const size_t kLdsBytes = 4 * TILE_ELEMS * sizeof(uint16_t);   // 65,536 bytes
 
 template <int EPI>
 static int launch(void* C, long ldc, const void* A, long lda, const void* W, long ldw, int M, int N, int K, int splits,
