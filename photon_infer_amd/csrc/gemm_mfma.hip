@@ -255,25 +255,27 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
   load_slab(0, 0);
   __builtin_amdgcn_s_waitcnt(0x0F70);       // vmcnt(0): this wave's pieces of the slab are in LDS
   __syncthreads();
+  load_slab(BK, 1);
   read_frags(0, 0, 0);
   for (int s = 0; s < slabs; ++s) {
     const int buf = s & 1;
-    load_slab((s + 1) * BK, buf ^ 1);       // into the buffer everybody left at the last barrier; beyond the range: zeros, unused
     read_frags(1, buf, 1);
     products(0);
-    PI_DEAL4(PI_SCHED_DS_READ, PI_SCHED_VMEM_READ)
+    PI_DEAL4(PI_SCHED_DS_READ, 0)
     read_frags(0, buf, 2);
     products(1);
     PI_DEAL4(PI_SCHED_DS_READ, 0)
     read_frags(1, buf, 3);
     products(0);
     PI_DEAL4(PI_SCHED_DS_READ, 0)
-    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __builtin_amdgcn_s_waitcnt(0x0F70);     // slab s + 1 has landed (asked for a whole slab ago)
     __syncthreads();
+    load_slab((s + 2) * BK, buf);           // into the buffer everybody has just left; beyond the range: zeros, unused
     read_frags(0, buf ^ 1, 0);
     products(1);
-    PI_DEAL4(PI_SCHED_DS_READ, 0)
+    PI_DEAL4(PI_SCHED_DS_READ, PI_SCHED_VMEM_READ)
   }
+  __builtin_amdgcn_s_waitcnt(0x0F70);       // nothing may still be on its way into LDS when the patches take it over
 #undef PI_DEAL4
   __syncthreads();                  // the fragments read last belong to no slab; LDS is free for the patches
 
@@ -405,13 +407,13 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
     if (kind_a) __builtin_amdgcn_sched_group_barrier(kind_a, 1, 0);                  \
     if (kind_b) __builtin_amdgcn_sched_group_barrier(kind_b, 1, 0);                  \
   }
+  load_slab(1, 1);
   for (int s = 0; s < slabs; ++s) {
     const int buf = s & 1;
-    load_slab(s + 1, buf ^ 1);      // into the buffer everybody left at the last barrier
     read_frags(1, buf, 1);
     products(0);
-    PI_DEAL(6, PI_SCHED_DS_READ, PI_SCHED_VMEM_READ)
-    PI_DEAL(2, PI_SCHED_VMEM_READ, 0)
+    PI_DEAL(6, PI_SCHED_DS_READ, 0)
+    PI_DEAL(2, 0, 0)
     read_frags(0, buf, 2);
     products(1);
     PI_DEAL(6, PI_SCHED_DS_READ, 0)
@@ -420,13 +422,15 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
     products(0);
     PI_DEAL(6, PI_SCHED_DS_READ, 0)
     PI_DEAL(2, 0, 0)
-    __builtin_amdgcn_s_waitcnt(0x0F70);
+    __builtin_amdgcn_s_waitcnt(0x0F70);     // slab s + 1 has landed (asked for a whole slab ago)
     __syncthreads();
+    load_slab(s + 2, buf);          // into the buffer everybody has just left
     read_frags(0, buf ^ 1, 0);
     products(1);
-    PI_DEAL(6, PI_SCHED_DS_READ, 0)
-    PI_DEAL(2, 0, 0)
+    PI_DEAL(6, PI_SCHED_DS_READ, PI_SCHED_VMEM_READ)
+    PI_DEAL(2, PI_SCHED_VMEM_READ, 0)
   }
+  __builtin_amdgcn_s_waitcnt(0x0F70);       // nothing may still be on its way into LDS when the patches take it over
 #undef PI_DEAL
 
   // acc[i][j][v] is C[m0 + wm*128 + i*32 + 8*(v/4) + 4*(lane/32) + v%4][n0 + wn*64 + j*32 + lane%32].
