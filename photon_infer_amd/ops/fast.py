@@ -22,6 +22,7 @@ from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
+from ..errors import KernelError
 from . import _lib
 from .workspace import GEMM_PART_FLOATS, KernelWorkspace, KeyRanges, Partials, PendingUpdate
 
@@ -35,6 +36,8 @@ SHARED_TARGET_BLOCKS = 256     # ... and this many blocks wanted (one per comput
 TILE_MAX_SPLITS = 4
 BIG_MIN_TILES = 192            # 256 x 256 tiles (times k pieces) from which the large-tile kernel is taken (the library's rule)
 BIG_MIN_K = 1024               # a piece of the large-tile kernel keeps at least this much of k
+BIG_SPLIT_MIN_K = 6144         # ... and k is cut for it only from this length on
+FULL_CHIP_TILES = 256          # from this many 128 x 128 tiles on (one per compute unit) k is not cut for them
 PIECES_BELOW_TILES = 200       # fewer 128 x 128 tiles than this: q, k, v of a prompt portion are left in k pieces too
 TILE_HEAD_DIMS = tuple(range(16, 257, 16))         # head sizes of the prompt-attention tile kernel (above 128: rounds of 64 keys, 16 columns per wave)
 DECODE_HEAD_DIMS = tuple(range(16, 257, 16))       # head sizes of the key-split decode kernel
@@ -71,11 +74,15 @@ def _tile_splits(M: int, N: int, K: int) -> int:
         # pieces on the large-tile kernel as give every compute unit one block (measured at
         # 2048 x 2048 x 8192: four pieces 72 us, against 87 us for two pieces on the small tiles,
         # and 6 us more in the norm that adds them)
+        # and k long enough that the faster kernel outweighs the pieces' way through memory: the
+        # o projection of such a prompt (k = 3,072 / 4,096, two pieces) took 68 / 93 us with its
+        # norm against 61 / 86 us unsplit on the small tiles
         for pieces in (4, 3, 2):
-            if BIG_MIN_TILES <= big * pieces <= 256 and K >= pieces * BIG_MIN_K and pieces * M * N <= GEMM_PART_FLOATS:
+            if (BIG_MIN_TILES <= big * pieces <= 256 and K >= max(pieces * BIG_MIN_K, BIG_SPLIT_MIN_K)
+                    and pieces * M * N <= GEMM_PART_FLOATS):
                 return pieces
     tiles = -(-M // 128) * -(-N // 128)
-    splits = min(TILE_MAX_SPLITS, TARGET_BLOCKS // max(1, tiles), K // 512)
+    splits = 1 if tiles >= FULL_CHIP_TILES else min(TILE_MAX_SPLITS, TARGET_BLOCKS // max(1, tiles), K // 512)
     while splits > 1 and splits * M * N > GEMM_PART_FLOATS:
         splits -= 1
     return max(1, splits)
@@ -95,6 +102,9 @@ def _piece_buffer(ws: Optional[KernelWorkspace], floats: int, device) -> torch.T
     applied first), or memory of this call's own."""
     if ws is None:
         return torch.empty(floats, dtype=torch.float32, device=device)
+    if floats > GEMM_PART_FLOATS:
+        # the split rules never ask for more; a kernel writing pieces past the buffer would fault the GPU
+        raise KernelError(f"pieces of a split product need {floats} floats, the workspace holds {GEMM_PART_FLOATS}")
     flush(ws)
     return ws.gemm_part
 

@@ -219,10 +219,11 @@ def test_gemm_on_large_tiles(_ops, M, N, K):
     close(acc, want + base.double(), 2e-6, "large gemm accumulate")
 
 
-def test_gemm_on_large_tiles_split_over_k(_ops):
-    """Few output tiles and a long k: pieces over k from the large-tile kernel, summed by materialize."""
+@pytest.mark.parametrize("M,N,K", [(2048, 2040, 6208),      # 64 tiles of 256 x 256, a long k: four pieces on the large-tile kernel
+                                   (1024, 2040, 4104)])     # 128 tiles of 128 x 128, k no multiple of the slab: pieces on the small tiles
+def test_gemm_on_large_tiles_split_over_k(_ops, M, N, K):
+    """Few output tiles and a long k: pieces over k from the tile kernels, summed by materialize."""
     _ops.use_fast_kernels(True)
-    M, N, K = 2048, 2040, 4104
     a = (torch.randn(M, K, generator=gen(1)) * 0.25).to(BF16)
     w = (torch.randn(N, K, generator=gen(2)) * 0.25).to(BF16)
     base = torch.randn(M, N, generator=gen(3))
