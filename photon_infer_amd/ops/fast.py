@@ -37,7 +37,6 @@ TILE_MAX_SPLITS = 4
 BIG_MIN_TILES = 192            # 256 x 256 tiles (times k pieces) from which the large-tile kernel is taken (the library's rule)
 BIG_MIN_K = 1024               # a piece of the large-tile kernel keeps at least this much of k
 BIG_SPLIT_MIN_K = 6144         # ... and k is cut for it only from this length on
-FULL_CHIP_TILES = 256          # from this many 128 x 128 tiles on (one per compute unit) k is not cut for them
 PIECES_BELOW_TILES = 200       # fewer 128 x 128 tiles than this: q, k, v of a prompt portion are left in k pieces too
 TILE_HEAD_DIMS = tuple(range(16, 257, 16))         # head sizes of the prompt-attention tile kernel (above 128: rounds of 64 keys, 16 columns per wave)
 DECODE_HEAD_DIMS = tuple(range(16, 257, 16))       # head sizes of the key-split decode kernel
@@ -82,7 +81,7 @@ def _tile_splits(M: int, N: int, K: int) -> int:
                     and pieces * M * N <= GEMM_PART_FLOATS):
                 return pieces
     tiles = -(-M // 128) * -(-N // 128)
-    splits = 1 if tiles >= FULL_CHIP_TILES else min(TILE_MAX_SPLITS, TARGET_BLOCKS // max(1, tiles), K // 512)
+    splits = min(TILE_MAX_SPLITS, TARGET_BLOCKS // max(1, tiles), K // 512)
     while splits > 1 and splits * M * N > GEMM_PART_FLOATS:
         splits -= 1
     return max(1, splits)
