@@ -99,3 +99,18 @@ def test_steps_of_single_tokens_need_no_plan_unless_the_tile_kernel_serves_them(
     arrays, _ = AttentionPlanner(16, 0, 2, False, 256).plan([1, 1, 1], [5, 900, 17])
     assert arrays["req"].tolist()[:3] == [0, 1, 2] or sorted(set(arrays["req"].tolist())) == [0, 1, 2]
     assert arrays["singles"].size == 0
+
+
+def test_pieces_that_would_not_fit_the_workspace_are_refused():
+    """The kernels write a split product's pieces without knowing the buffer's size: the host
+    refuses a request beyond it, and the split rules never make one."""
+    from photon_infer_amd.errors import KernelError
+    from photon_infer_amd.ops import fast
+    from photon_infer_amd.ops.workspace import GEMM_PART_FLOATS, KernelWorkspace
+    with pytest.raises(KernelError, match="workspace holds"):
+        fast._piece_buffer(KernelWorkspace("cpu"), GEMM_PART_FLOATS + 1, "cpu")
+    for M, N, K in [(2048, 2048, 8192), (2048, 3072, 8192), (2048, 4096, 14336), (8192, 4096, 14336), (4096, 8192, 28672),
+                    (512, 4096, 14336), (100000, 128, 4096), (129, 128256, 2048)]:
+        assert fast._tile_splits(M, N, K) * M * N <= GEMM_PART_FLOATS or fast._tile_splits(M, N, K) == 1
+    for M, N, K in [(8, 128256, 2048), (128, 128256, 8192), (64, 16384, 2048), (1, 2048, 8192)]:
+        assert fast._skinny_splits(M, N, K) * M * N <= GEMM_PART_FLOATS or fast._skinny_splits(M, N, K) == 1
