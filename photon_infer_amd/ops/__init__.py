@@ -59,7 +59,7 @@ def _gpu(*tensors: Optional[torch.Tensor]) -> None:
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    return _lib.current_stream()
 
 
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:

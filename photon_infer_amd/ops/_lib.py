@@ -3,7 +3,9 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_float, c_int, c_long, c_void_p
-from typing import Dict
+from typing import Dict, Optional
+
+import torch
 
 from ..errors import KernelError, KernelLibraryMissing
 from . import build
@@ -38,6 +40,22 @@ _SIGNATURES = {
 }
 
 _LIBS: Dict[str, ctypes.CDLL] = {}
+
+
+_RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_DEVICE_INDEX: Optional[int] = None
+
+
+def current_stream() -> int:
+    """The current HIP stream's handle.  Asked for at every kernel launch (a step of a few
+    hundred launches), so by the shortest way torch offers: its Python-level
+    ``current_stream()`` costs as much as the launch itself."""
+    global _DEVICE_INDEX
+    if _RAW_STREAM is None:
+        return torch.cuda.current_stream().cuda_stream
+    if _DEVICE_INDEX is None:
+        _DEVICE_INDEX = torch.cuda.current_device()      # one process, one GPU
+    return _RAW_STREAM(_DEVICE_INDEX)
 
 
 def load(module: str) -> ctypes.CDLL:

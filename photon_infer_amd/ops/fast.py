@@ -47,7 +47,7 @@ DECODE_MIN_KEYS_PER_SPLIT = 128
 
 
 def _stream() -> int:
-    return torch.cuda.current_stream().cuda_stream
+    return _lib.current_stream()
 
 
 def _gemm_ok(a, w, K, lda, ldw) -> bool:
