@@ -183,7 +183,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
     for (int t = 0; t < RT; ++t)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        w[t][h] = load_frag(wrow[t] + (whole || kk + lg * 16 + h * 8 < k1 ? kk + h * 8 : k0));
+        // a piece beyond k1 is fetched from the range's first 8 elements instead (k0 + 8 <= k1:
+        // both are multiples of 8), which lie inside the row whatever the lane's own offset
+        w[t][h] = load_frag(wrow[t] + (whole || kk + lg * 16 + h * 8 < k1 ? kk + h * 8 : k0 - lg * 16));
         if (!whole && kk + lg * 16 + h * 8 >= k1) w[t][h] = zero_frag();
       }
     if constexpr (RANGES) {
@@ -206,7 +208,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
 #pragma unroll
       for (int i = 0; i < MB * 2; ++i)
         if (i == 0 || i < x_loads) {
-          xg[i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + (x_ok ? kk : k0));
+          xg[i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + (x_ok ? kk : k0 - xp * 8));
           if (!x_ok) xg[i] = u32x4_t{0u, 0u, 0u, 0u};
         }
 #pragma unroll

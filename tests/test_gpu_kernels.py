@@ -158,7 +158,9 @@ def test_swiglu(_ops, dtype):
 # ------------------------------------------------------------------ matrix products
 GEMM_SHAPES = [(1, 14, 3), (2, 2, 3), (5, 176, 64), (33, 100, 72), (64, 384, 128), (70, 1001, 96), (1, 256, 64),
                (130, 64, 200), (257, 320, 136), (8, 2048, 512), (300, 520, 264),
-               (40, 200, 1032), (64, 72, 520), (48, 1001, 96), (35, 130, 2048)]
+               (40, 200, 1032), (64, 72, 520), (48, 1001, 96), (35, 130, 2048),
+               # few rows and a k of which some wave holds less than one step of 64
+               (4, 50, 160), (16, 33, 8), (3, 64, 200), (9, 40, 344), (12, 776, 272)]
 
 
 @pytest.mark.parametrize("M,N,K", GEMM_SHAPES)
