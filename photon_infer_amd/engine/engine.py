@@ -21,12 +21,11 @@ from .step import ModelRunner, StepEntry
 class _InFlight:
     """A decode step that runs on the GPU while the host goes on."""
 
-    def __init__(self, reqs: List[InferenceRequest], ids, host):
-        import torch
+    def __init__(self, reqs: List[InferenceRequest], ids, host, done):
         self.reqs = reqs            # in the order of the step's rows
         self.ids = ids              # the step's tokens on the device
         self.host = host            # pinned buffer they are copied to
-        self.done = torch.cuda.Event()
+        self.done = done            # event recorded behind the copy
         self.ended: List[InferenceRequest] = []   # requests in this step that had already ended when it was launched
 
 
@@ -124,19 +123,18 @@ class ContinuousBatchEngine:
         temps = [r.params.temperature for r in reqs]
         draws = [uniform_draw(r.params.seed, r.num_generated() + pending) if r.params.temperature > 0 else 0.0 for r in reqs]
         ids = self.runner.decode_step(entries, temps, draws, feed)
-        fl = _InFlight(reqs, ids, self._token_buffer(len(reqs)))
+        fl = _InFlight(reqs, ids, self._token_buffer(len(reqs)), self.runner.new_event())
         fl.host.copy_(ids, non_blocking=True)
         fl.done.record()
         self._in_flight = fl
         self.steps += 1
 
     def _token_buffer(self, n: int):
-        import torch
         # two pinned buffers per size, used in turn: one is still being read when the next copy starts
         key = (n, self.steps % 2)
         buf = self._buffers.get(key)
         if buf is None:
-            buf = self._buffers[key] = torch.empty(n, dtype=torch.int32, pin_memory=True)
+            buf = self._buffers[key] = self.runner.host_token_buffer(n)
         return buf
 
     def _collect(self, fl: "_InFlight", skip: Sequence[InferenceRequest] = ()) -> List[InferenceRequest]:

@@ -241,6 +241,14 @@ class ModelRunner:
 
     graphs_captured = 0
 
+    # what a caller that reads a step's tokens later needs: an event to record behind its copy
+    # and page-locked memory to copy into
+    def new_event(self):
+        return torch.cuda.Event()
+
+    def host_token_buffer(self, n: int) -> torch.Tensor:
+        return torch.empty(n, dtype=torch.int32, pin_memory=True)
+
     def capture_stream(self):
         if getattr(self, "_capture_stream", None) is None:
             self._capture_stream = torch.cuda.Stream(device=self.device)
