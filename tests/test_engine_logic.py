@@ -60,13 +60,14 @@ class StandInRunner:
 
     graph_safe = True
 
-    def __init__(self, options: EngineOptions, max_model_len: int):
+    def __init__(self, options: EngineOptions, max_model_len: int, windows=(None,)):
         self.options = options
         self.max_model_len = max_model_len
         self.device = "cpu"
         self.workspace = None
         self.spec = types.SimpleNamespace(eos_token_ids=(END,), vocab_size=VOCAB)
-        self.cache = CacheManager([None], options.block_size, options.num_blocks, options.max_batch, max_model_len)
+        # one cache group per entry: all keys, or a window whose pages return while the request runs
+        self.cache = CacheManager(list(windows), options.block_size, options.num_blocks, options.max_batch, max_model_len)
         self.history = {}            # rid -> the tokens in the cache, by position
         self._results = {}           # batch size -> the one buffer every step of that size writes
         self.decode_steps = self.mixed_steps = self.fed_steps = 0
@@ -133,7 +134,7 @@ def make_engine(rng, lookahead, use_graphs, max_model_len=96):
     options = EngineOptions(block_size=page, num_blocks=rng.choice([6, 10, 16, 40, 200]), max_batch=rng.choice([1, 2, 3, 4, 6]),
                             max_step_tokens=rng.choice([4, 8, 16, 64]), chunk_size=rng.choice([2, 4, 8, 32]),
                             lookahead=lookahead, use_graphs=use_graphs, device="cpu")
-    runner = StandInRunner(options, max_model_len)
+    runner = StandInRunner(options, max_model_len, rng.choice([(None,), (None,), (None, 12), (20, None, 6)]))
     eng = ContinuousBatchEngine(None, runner=runner)
     eng.sampler = StandInSampler()
     return eng
@@ -200,7 +201,8 @@ def test_random_workloads_give_every_request_its_own_tokens(lookahead, use_graph
                 continue
             assert got == want and req.finish_reason == reason, f"{what}: request {i}: {got} != {want} ({req.finish_reason} / {reason})"
             ended_early += reason == "eos"
-        assert eng.runner.cache.num_live == 0 and eng.runner.cache.free_pages(0) == eng.options.num_blocks, what
+        assert eng.runner.cache.num_live == 0, what
+        assert all(eng.runner.cache.free_pages(g) == eng.options.num_blocks for g in range(len(eng.runner.cache.groups))), what
         assert not eng.runner.history, what
         fed += eng.runner.fed_steps
         preempted += eng.get_stats().num_preemptions
