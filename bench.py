@@ -413,6 +413,7 @@ def main() -> int:
             "tied_embeddings": cfg.tie_word_embeddings, "rope": "llama3 theta=500000 factor=32",
             "global_batch": args.batch, "seq_len": CONTEXT, "kv_block": BLOCK_SIZE, "prefill_tokens": PREFILL_TOKENS,
             "parallelism": "single-gpu", "weight_bytes": wbytes, "kv_bytes_per_token": kvb,
+            "weight_copies_in_streaming_order": runner.stream_copies,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},

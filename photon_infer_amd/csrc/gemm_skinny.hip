@@ -126,7 +126,7 @@ union SkinnyLds {
 template <int MB, int EPI, bool RANGES = false, int RT = 2>
 __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ X, long ldx,
                                                           const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
-                                                          int k_per_block, float* __restrict__ part, RangeSource rs) {
+                                                          int k_per_block, float* __restrict__ part, RangeSource rs, int tiled) {
   constexpr int ROWS = RT * 16;          // weight rows of a block: RT row tiles per wave
   static_assert(EPI != EPI_SWIGLU || RT == 2, "the SwiGLU epilogue pairs a wave's two row tiles");
   __shared__ SkinnyLds<MB, RT> lds;
@@ -143,10 +143,16 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
   const int k0 = kb0 + wave * per_wave;
   const int k1 = min(kb1, k0 + per_wave);
 
-  // rows beyond N read the last valid row; their results are never stored
+  // rows beyond N read the last valid row; their results are never stored.  `tiled`: W is the
+  // copy in the order this kernel reads (see pi_gemm_skinny): 16 rows x 64 k are 2 KB in a row,
+  // one load instruction's 1 KB after the other, so a k step of 64 moves by 1,024 elements and
+  // the step's second fragment lies 512 elements behind the first.
+  const int k_mul = tiled ? 16 : 1, h_mul = tiled ? 512 : 8;
   const bf16_t* wrow[RT];
 #pragma unroll
-  for (int t = 0; t < RT; ++t) wrow[t] = W + min(n0 + t * 16 + lr, (long)N - 1) * ldw + lg * 16;
+  for (int t = 0; t < RT; ++t)
+    wrow[t] = tiled ? W + min(n0 / 16 + t, (long)N / 16 - 1) * (K / 64) * 1024 + lg * 128 + lr * 8
+                    : W + min(n0 + t * 16 + lr, (long)N - 1) * ldw + lg * 16;
 
   // Activations of a k step: load instruction i brings tokens 8i .. 8i+7, lane j the 16-byte
   // piece j % 8 of token 8i + j / 8.  Tokens beyond M are not loaded: what LDS holds for them
@@ -185,7 +191,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
       for (int h = 0; h < 2; ++h) {
         // a piece beyond k1 is fetched from the range's first 8 elements instead (k0 + 8 <= k1:
         // both are multiples of 8), which lie inside the row whatever the lane's own offset
-        w[t][h] = load_frag(wrow[t] + (whole || kk + lg * 16 + h * 8 < k1 ? kk + h * 8 : k0 - lg * 16));
+        // (a tiled matrix has whole steps only)
+        if (whole) w[t][h] = load_frag(wrow[t] + (long)kk * k_mul + h * h_mul);
+        else w[t][h] = load_frag(wrow[t] + (kk + lg * 16 + h * 8 < k1 ? kk + h * 8 : k0 - lg * 16));
         if (!whole && kk + lg * 16 + h * 8 >= k1) w[t][h] = zero_frag();
       }
     if constexpr (RANGES) {
@@ -292,7 +300,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
 template <int MB, int EPI, int DEPTH>
 __global__ __launch_bounds__(256) void gemm_skinny_shared_kernel(void* __restrict__ Cv, long ldc, const bf16_t* __restrict__ X, long ldx,
                                                                  const bf16_t* __restrict__ W, long ldw, int M, int N, int K,
-                                                                 int k_per_block, float* __restrict__ part) {
+                                                                 int k_per_block, float* __restrict__ part, int tiled) {
   constexpr int ROWS = SHARED_ROWS_PER_BLOCK;
   constexpr int XL = (MB + 1) / 2;      // 16-byte pieces of an activation tile per lane
   __shared__ union {
@@ -309,7 +317,8 @@ __global__ __launch_bounds__(256) void gemm_skinny_shared_kernel(void* __restric
   auto k_of = [&](const int s) { return kb0 + min(s, steps - 1) * KSTEP; };   // steps beyond the last are fetched, never used
 
   // rows beyond N and tokens beyond M read the last valid one; their results are never stored
-  const bf16_t* wrow = W + min(n0 + wave * 16 + lr, (long)N - 1) * ldw;
+  const bf16_t* wrow = tiled ? W + min(n0 / 16 + wave, (long)N / 16 - 1) * (K / 64) * 1024 + lg * 128 + lr * 8     // see gemm_skinny_kernel
+                             : W + min(n0 + wave * 16 + lr, (long)N - 1) * ldw;
   const int xp = tid % 8;
   const bf16_t* xsrc[XL];
   int xdst[XL];
@@ -340,7 +349,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_shared_kernel(void* __restric
 #pragma unroll
     for (int i = 0; i < XL; ++i) xq[j][i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + min(kk + xp * 8, kb1 - 8));
 #pragma unroll
-    for (int h = 0; h < 2; ++h) wq[j][h] = load_frag(wrow + min(kk + lg * 16 + h * 8, kb1 - 8));
+    for (int h = 0; h < 2; ++h) wq[j][h] = load_frag(wrow + (tiled ? (long)kk * 16 + h * 512 : (long)min(kk + lg * 16 + h * 8, kb1 - 8)));
   };
 #pragma unroll
   for (int j = 0; j < DEPTH; ++j) fetch(j, j);
@@ -439,8 +448,8 @@ extern "C" int pi_splitk_reduce(void* C, int epilogue, long ldc, const void* par
 
 template <int MB>
 static int launch_mb(int epi, dim3 grid, hipStream_t stream, void* C, long ldc, const bf16_t* X, long ldx, const bf16_t* W,
-                     long ldw, int M, int N, int K, int kpb, float* part) {
-#define GO(E) hipLaunchKernelGGL((gemm_skinny_kernel<MB, E>), grid, dim3(256), 0, stream, C, ldc, X, ldx, W, ldw, M, N, K, kpb, part, RangeSource{})
+                     long ldw, int M, int N, int K, int kpb, float* part, int tiled) {
+#define GO(E) hipLaunchKernelGGL((gemm_skinny_kernel<MB, E>), grid, dim3(256), 0, stream, C, ldc, X, ldx, W, ldw, M, N, K, kpb, part, RangeSource{}, tiled)
   switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
     case EPI_F32: GO(EPI_F32); break;
@@ -454,8 +463,8 @@ static int launch_mb(int epi, dim3 grid, hipStream_t stream, void* C, long ldc, 
 
 template <int MB>
 static int launch_shared(int epi, dim3 grid, hipStream_t stream, void* C, long ldc, const bf16_t* X, long ldx, const bf16_t* W,
-                         long ldw, int M, int N, int K, int kpb, float* part) {
-#define GO(E) hipLaunchKernelGGL((gemm_skinny_shared_kernel<MB, E, SHARED_DEPTH>), grid, dim3(256), 0, stream, C, ldc, X, ldx, W, ldw, M, N, K, kpb, part)
+                         long ldw, int M, int N, int K, int kpb, float* part, int tiled) {
+#define GO(E) hipLaunchKernelGGL((gemm_skinny_shared_kernel<MB, E, SHARED_DEPTH>), grid, dim3(256), 0, stream, C, ldc, X, ldx, W, ldw, M, N, K, kpb, part, tiled)
   switch (epi) {
     case EPI_BF16: GO(EPI_BF16); break;
     case EPI_F32: GO(EPI_F32); break;
@@ -472,8 +481,15 @@ extern "C" int pi_gemm_skinny_rows_per_block(int M) { return M > SHARED_FROM_TOK
 
 // splits > 1: the partial products go to `part` (float32 [splits, M, N]) and C is not touched;
 // *splits_out tells how many splits were made (no empty ones).
+// `tiled` != 0: W is not [N, K] row after row but a copy in the order the kernels' loads want it,
+// [N / 16][K / 64][2][4][16][8]: for 16 rows and 64 k, first the k of every lane's first
+// fragment, then of its second; in each, lane group g's k = 16 g + 8 h .. + 7 of rows 0..15.
+// A wave's load instruction then reads 1 KB in a row instead of 64 bytes from each of 16 rows.
+// N must be a multiple of 16 and K of 64.
 extern "C" int pi_gemm_skinny(void* C, int epilogue, long ldc, const void* X, long ldx, const void* W, long ldw, int M,
-                              int N, int K, int splits, void* part, long part_elems, int* splits_out, hipStream_t stream) {
+                              int N, int K, int splits, void* part, long part_elems, int* splits_out, int tiled,
+                              hipStream_t stream) {
+  PI_REQUIRE(!tiled || (N % 16 == 0 && K % 64 == 0), "gemm_skinny: a tiled weight matrix needs N (%d) a multiple of 16 and K (%d) of 64", N, K);
   PI_REQUIRE(M > 0 && M <= 128 && N > 0 && K > 0, "gemm_skinny: takes 1..128 rows, got M=%d N=%d K=%d", M, N, K);
   PI_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, "gemm_skinny: K (%d) and row strides (%ld, %ld) must be multiples of 8", K, ldx, ldw);
   PI_REQUIRE(((uintptr_t)X % 16 == 0) && ((uintptr_t)W % 16 == 0), "gemm_skinny: operands must be 16-byte aligned");
@@ -490,18 +506,18 @@ extern "C" int pi_gemm_skinny(void* C, int epilogue, long ldc, const void* X, lo
   const int mb = (M + 15) / 16;
   const bf16_t *x = (const bf16_t*)X, *w = (const bf16_t*)W;
   if (M > SHARED_FROM_TOKENS) {
-#define SHARED(B) case B: return launch_shared<B>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part)
+#define SHARED(B) case B: return launch_shared<B>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part, tiled)
     switch (mb) {
       SHARED(3); SHARED(4); SHARED(5); SHARED(6); SHARED(7);
-      default: return launch_shared<8>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
+      default: return launch_shared<8>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part, tiled);
     }
 #undef SHARED
   }
   switch (mb) {
-    case 1: return launch_mb<1>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
-    case 2: return launch_mb<2>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
-    case 3: return launch_mb<3>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
-    default: return launch_mb<4>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part);
+    case 1: return launch_mb<1>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part, tiled);
+    case 2: return launch_mb<2>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part, tiled);
+    case 3: return launch_mb<3>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part, tiled);
+    default: return launch_mb<4>(epilogue, grid, stream, C, ldc, x, ldx, w, ldw, M, N, K, kpb, (float*)part, tiled);
   }
 }
 
@@ -511,7 +527,7 @@ extern "C" int pi_gemm_skinny(void* C, int epilogue, long ldc, const void* X, lo
 // belong to one head.  Epilogues: store bf16, store f32, add into f32.
 extern "C" int pi_gemm_skinny_ranges(void* C, int epilogue, long ldc, const void* ranges, int heads, int head_dim, int count,
                                      const void* W, long ldw, int M, int N, int splits, void* part, long part_elems,
-                                     int* splits_out, hipStream_t stream) {
+                                     int* splits_out, int tiled, hipStream_t stream) {
   PI_REQUIRE(M > 0 && M <= 16 && N > 0 && heads > 0 && count >= 1 && count <= 64, "gemm_skinny_ranges: takes 1..16 tokens and 1..64 ranges, got M=%d N=%d heads=%d ranges=%d", M, N, heads, count);
   PI_REQUIRE(head_dim > 0 && head_dim % KSTEP == 0, "gemm_skinny_ranges: head_dim %d is no multiple of %d", head_dim, KSTEP);
   PI_REQUIRE(epilogue == EPI_BF16 || epilogue == EPI_F32 || epilogue == EPI_ACCUM, "gemm_skinny_ranges: unknown epilogue %d", epilogue);
@@ -519,6 +535,7 @@ extern "C" int pi_gemm_skinny_ranges(void* C, int epilogue, long ldc, const void
   PI_REQUIRE(splits >= 1 && splits <= 65535, "gemm_skinny_ranges: bad split count %d", splits);
   const long K = (long)heads * head_dim;
   PI_REQUIRE(K < (1L << 30), "gemm_skinny_ranges: k too long");
+  PI_REQUIRE(!tiled || N % 16 == 0, "gemm_skinny_ranges: a tiled weight matrix needs N (%d) a multiple of 16", N);
   int kpb = ceil_div((int)K, splits);
   kpb = ((kpb + 4 * KSTEP - 1) / (4 * KSTEP)) * (4 * KSTEP);     // a block's four waves take whole steps
   splits = ceil_div((int)K, kpb);
@@ -528,7 +545,7 @@ extern "C" int pi_gemm_skinny_ranges(void* C, int epilogue, long ldc, const void
   const dim3 grid(ceil_div(N, RANGES_ROW_TILES * 16), splits);
   const RangeSource rs{(const float*)ranges, heads, head_dim, count};
 #define GO(E) hipLaunchKernelGGL((gemm_skinny_kernel<1, E, true, RANGES_ROW_TILES>), grid, dim3(256), 0, stream, C, ldc, (const bf16_t*)nullptr, 0L, \
-                                 (const bf16_t*)W, ldw, M, N, (int)K, kpb, (float*)part, rs)
+                                 (const bf16_t*)W, ldw, M, N, (int)K, kpb, (float*)part, rs, tiled)
   switch (epilogue) {
     case EPI_BF16: GO(EPI_BF16); break;
     case EPI_F32: GO(EPI_F32); break;

@@ -65,6 +65,15 @@ class ModelRunner:
         # runner's own, handed to the parts with every step's context
         self.workspace = ops.KernelWorkspace(self.device)
         self.workspace.prepare(self.dtype == torch.bfloat16 and ops.fast_kernels_enabled())
+        # a second copy of the matrices that every decode step streams, in the order the kernels
+        # read them; made before the cache is sized, which takes what memory is left
+        self.stream_copies = 0
+        if self.options.stream_copies and self.dtype == torch.bfloat16 and ops.fast_kernels_enabled():
+            seen = set()
+            for w in self.model.streamed_weights():
+                if w is not None and w.data_ptr() not in seen:       # a tied head names the embedding's matrix
+                    seen.add(w.data_ptr())
+                    self.stream_copies += int(self.workspace.add_stream_copy(w))
         self._build_cache()
         # what the mixers want planned on the host per step (equal planners are kept once)
         self.planners = []

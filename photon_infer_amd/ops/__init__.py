@@ -17,7 +17,7 @@ import torch
 
 from ..errors import KernelError
 from . import _lib
-from .workspace import KernelWorkspace, KeyRanges, Partials
+from .workspace import KernelWorkspace, KeyRanges, Partials, stream_layout
 
 PI_F32, PI_BF16 = 0, 1
 MAX_HEAD_DIM = 256
@@ -181,7 +181,7 @@ def gemm_swiglu(out: torch.Tensor, a: torch.Tensor, w_gate_up: torch.Tensor, blo
         return
     if _FAST and block == 16 and a.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16 and out.is_contiguous():
         from . import fast
-        if fast.gemm_swiglu(out, a, w_gate_up, M, 2 * I, a.shape[1], _rows(a, "gemm a"), _rows(w_gate_up, "gemm w")):
+        if fast.gemm_swiglu(out, a, w_gate_up, M, 2 * I, a.shape[1], _rows(a, "gemm a"), _rows(w_gate_up, "gemm w"), ws):
             return
     gu = torch.empty((M, 2 * I), dtype=a.dtype, device=a.device)
     gemm(gu, a, w_gate_up, ws=ws)

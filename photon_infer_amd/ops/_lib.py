@@ -28,14 +28,14 @@ _SIGNATURES = {
     "bf16": {
         "pi_gemm_mfma": [P, I, L, P, L, P, L, I, I, I, I, P],
         "pi_gemm_mfma_pieces": [I, I],
-        "pi_gemm_skinny": [P, I, L, P, L, P, L, I, I, I, I, P, L, P, P],
+        "pi_gemm_skinny": [P, I, L, P, L, P, L, I, I, I, I, P, L, P, I, P],
         "pi_splitk_reduce": [P, I, L, P, I, I, I, P],
         "pi_attention_tile_rows": [I, I, I],
         "pi_attention_prefill_mfma": [P, L, P, L, P, P, P, I, P, P, P, P, P, P, P, P, I, I, I, I, I, I, F, I, L, P],
         "pi_attention_combine_rows": [P, L, P, I, P, I, I, I, P],
         "pi_attention_decode": [P, L, P, L, P, P, P, I, P, P, P, I, I, I, I, I, F, I, L, I, P, L, P],
         "pi_attention_decode_fused": [P, L, P, L, P, I, I, I, P, I, P, P, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, I, P],
-        "pi_gemm_skinny_ranges": [P, I, L, P, I, I, I, P, L, I, I, I, P, L, P, P],
+        "pi_gemm_skinny_ranges": [P, I, L, P, I, I, I, P, L, I, I, I, P, L, P, I, P],
     },
 }
 

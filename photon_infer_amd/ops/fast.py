@@ -108,13 +108,25 @@ def _piece_buffer(ws: Optional[KernelWorkspace], floats: int, device) -> torch.T
     return ws.gemm_part
 
 
+def _streamed(ws: Optional[KernelWorkspace], w, N: int, K: int, ldw: int):
+    """(address, tiled) of the weight matrix for the weight-streaming kernels: its copy in their
+    own order when the workspace keeps one, else the matrix itself."""
+    if ws is not None and ws.stream_copies and ldw == K:
+        copy = ws.stream_copy_of(w, N, K)
+        if copy is not None:
+            return copy.data_ptr(), 1
+    return w.data_ptr(), 0
+
+
 def _skinny(out_ptr: int, epilogue: int, ldc: int, a, w, M, N, K, lda, ldw, splits: int,
-            ws: Optional[KernelWorkspace]) -> Optional[Partials]:
-    """Run the weight-streaming kernel; returns the pieces when the product was split."""
-    buf = _piece_buffer(ws, splits * M * N, a.device) if splits > 1 else None
+            ws: Optional[KernelWorkspace], pieces_ws: bool = True) -> Optional[Partials]:
+    """Run the weight-streaming kernel; returns the pieces when the product was split.
+    ``pieces_ws`` False: the workspace is only asked for the weights' streaming copy."""
+    buf = _piece_buffer(ws if pieces_ws else None, splits * M * N, a.device) if splits > 1 else None
     made = ctypes.c_int(0)
-    _lib.call("bf16", "pi_gemm_skinny", out_ptr, epilogue, ldc, a.data_ptr(), lda, w.data_ptr(), ldw, M, N, K, splits,
-              None if buf is None else buf.data_ptr(), 0 if buf is None else buf.numel(), ctypes.byref(made), _stream())
+    w_ptr, tiled = _streamed(ws, w, N, K, ldw)
+    _lib.call("bf16", "pi_gemm_skinny", out_ptr, epilogue, ldc, a.data_ptr(), lda, w_ptr, ldw, M, N, K, splits,
+              None if buf is None else buf.data_ptr(), 0 if buf is None else buf.numel(), ctypes.byref(made), tiled, _stream())
     if made.value > 1:
         if ws is not None:
             ws.counts["split_products"] += 1
@@ -208,9 +220,10 @@ def gemm_from_ranges(out, kr: KeyRanges, w, accumulate, N, ldw, ldc, may_defer, 
     splits = _skinny_splits(M, N, K)
     buf = _piece_buffer(ws, splits * M * N, w.device) if splits > 1 else None
     made = ctypes.c_int(0)
+    w_ptr, tiled = _streamed(ws, w, N, K, ldw)
     _lib.call("bf16", "pi_gemm_skinny_ranges", out.data_ptr(), epilogue, ldc, kr.part.data_ptr(), kr.heads, kr.head_dim, kr.count,
-              w.data_ptr(), ldw, M, N, splits, None if buf is None else buf.data_ptr(), 0 if buf is None else buf.numel(),
-              ctypes.byref(made), _stream())
+              w_ptr, ldw, M, N, splits, None if buf is None else buf.data_ptr(), 0 if buf is None else buf.numel(),
+              ctypes.byref(made), tiled, _stream())
     if ws is not None:
         ws.counts["ranges_merged_by_product"] += 1
     if made.value > 1:
@@ -250,7 +263,7 @@ def gemm_pieces(a, w, ws: Optional[KernelWorkspace]) -> Optional[Partials]:
     return _skinny(0, EPI_F32, N, a, w, M, N, K, lda, ldw, splits, ws)
 
 
-def gemm_swiglu(out, a, w, M, N, K, lda, ldw) -> bool:
+def gemm_swiglu(out, a, w, M, N, K, lda, ldw, ws: Optional[KernelWorkspace] = None) -> bool:
     """``w`` [N = 2I, K] with gate / up rows interleaved in blocks of 16; out [M, I] bfloat16."""
     if not _gemm_ok(a, w, K, lda, ldw) or N % 32 or out.dtype != torch.bfloat16:
         return False
@@ -258,7 +271,7 @@ def gemm_swiglu(out, a, w, M, N, K, lda, ldw) -> bool:
         _lib.call("bf16", "pi_gemm_mfma", out.data_ptr(), EPI_SWIGLU, out.stride(0), a.data_ptr(), lda, w.data_ptr(), ldw,
                   M, N, K, 1, _stream())
     else:
-        _skinny(out.data_ptr(), EPI_SWIGLU, out.stride(0), a, w, M, N, K, lda, ldw, 1, None)
+        _skinny(out.data_ptr(), EPI_SWIGLU, out.stride(0), a, w, M, N, K, lda, ldw, 1, ws, pieces_ws=False)
     return True
 
 

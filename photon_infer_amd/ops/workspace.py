@@ -11,7 +11,7 @@ from __future__ import annotations
 
 from collections import Counter
 from dataclasses import dataclass
-from typing import Optional
+from typing import Dict, Optional, Tuple
 
 import torch
 
@@ -61,6 +61,20 @@ class PendingUpdate:
         return t is x or (t.data_ptr() == x.data_ptr() and t.shape == x.shape and t.stride() == x.stride())
 
 
+def stream_layout(w: torch.Tensor) -> Optional[torch.Tensor]:
+    """The bfloat16 matrix ``w`` [N, K] (N a multiple of 16, K of 64, rows contiguous) as
+    [N / 16][K / 64][2][4][16][8]: for every 16 rows and 64 columns, the 1 KB that a wave of the
+    weight-streaming kernels loads with one instruction lies in a row (lane group g of a wave
+    holds columns 16 g + 8 h .. + 7 of its row in its fragment h).  None for other matrices."""
+    if w.dim() != 2 or w.dtype != torch.bfloat16 or not w.is_contiguous():
+        return None
+    N, K = w.shape
+    if N == 0 or N % 16 or K == 0 or K % 64:
+        return None
+    tiles = w.view(N // 16, 16, K // 64, 4, 2, 8)          # [row block, row, k block, lane group, fragment, 8 columns]
+    return tiles.permute(0, 2, 4, 3, 1, 5).contiguous().view(N, K)
+
+
 class KernelWorkspace:
     """Buffers are made at first use and kept; ``counts`` says which paths a step took (tests
     read it: ``split_products``, ``deferred``, ``added_by_norm``, ``applied``, ``flushed``,
@@ -74,6 +88,9 @@ class KernelWorkspace:
         self._sample_part: Optional[torch.Tensor] = None
         self.pending: Optional[PendingUpdate] = None
         self.counts: Counter = Counter()
+        # weight matrices that have a second copy in the order the weight-streaming kernels read
+        # (steps of up to 128 tokens): address of the matrix -> (copy, rows, columns)
+        self.stream_copies: Dict[int, Tuple[torch.Tensor, int, int]] = {}
 
     def _buffer(self, name: str, floats: int) -> torch.Tensor:
         buf = getattr(self, name)
@@ -104,6 +121,22 @@ class KernelWorkspace:
         if matrix_core_kernels:
             self.gemm_part
             self.attn_part
+
+    def add_stream_copy(self, w: torch.Tensor) -> bool:
+        """Keep a copy of the bfloat16 matrix ``w`` [N, K] in the weight-streaming kernels' order
+        (``stream_layout``); products of up to 128 tokens with ``w`` then read the copy.  False,
+        and nothing kept, for a matrix whose sizes the layout does not take."""
+        copy = stream_layout(w)
+        if copy is None:
+            return False
+        self.stream_copies[w.data_ptr()] = (copy, w.shape[0], w.shape[1])
+        return True
+
+    def stream_copy_of(self, w: torch.Tensor, N: int, K: int) -> Optional[torch.Tensor]:
+        entry = self.stream_copies.get(w.data_ptr())
+        if entry is None or entry[1] != N or entry[2] != K:
+            return None
+        return entry[0]
 
     def take_pending(self, x: torch.Tensor) -> Optional[Partials]:
         """The pieces still to be added to ``x``, if any; they are the caller's to add."""

@@ -91,6 +91,9 @@ class PagedAttention(Mixer):
             own = {n[len(POSITION_PREFIX):]: t for n, t in tensors.items() if n.startswith(POSITION_PREFIX)}
             self.position.load(own, dtype, device)
 
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [self.w_qkv, self.w_o]
+
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
         T = h.shape[0]
         writes = self.own_kv and cache.writes

@@ -113,6 +113,13 @@ class Part:
         self.dtype = dtype
         self.device = device
 
+    def streamed_weights(self) -> List[torch.Tensor]:
+        """After ``load``: the weight matrices [out, in] that this part hands to ``ops.gemm`` /
+        ``ops.gemm_swiglu`` whole, in every decode step.  Whoever runs the model may keep a second
+        copy of each in the order the weight-streaming kernels read (``EngineOptions.stream_copies``);
+        a part that names none loses nothing but that."""
+        return []
+
 
 class Norm(Part):
     def forward(self, x: torch.Tensor, ctx: Optional[StepContext] = None, rows: Optional[torch.Tensor] = None) -> torch.Tensor:

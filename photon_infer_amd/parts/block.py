@@ -35,6 +35,9 @@ class PreNormBlock(Block):
     def graph_safe(self) -> bool:
         return all(part.graph_safe for _, part in self._named)
 
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [w for _, part in self._named for w in part.streamed_weights()]
+
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
         # A mixer or feed-forward may leave its update of x in pieces for the next norm to add
         # (ops.gemm(..., may_defer=True)).  A norm that does not go through ops.rmsnorm gets

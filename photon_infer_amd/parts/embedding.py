@@ -54,6 +54,9 @@ class LMHead(Part):
         super().load(tensors, dtype, device)
         self.weight = tied_weight if self.tied else tensors["weight"]
 
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [self.weight]
+
     def forward(self, h: torch.Tensor, ctx=None) -> torch.Tensor:
         """activations [M, hidden] -> float32 logits [M, vocab]."""
         logits = torch.empty((h.shape[0], self.vocab_size), dtype=torch.float32, device=h.device)

@@ -54,6 +54,9 @@ class SwiGLU(FeedForward):
             self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
         self.w_down = tensors["down_proj.weight"]
 
+    def streamed_weights(self) -> List[torch.Tensor]:
+        return [self.w_gate_up, self.w_down]
+
     def forward(self, h: torch.Tensor, x: torch.Tensor, ctx: StepContext) -> None:
         act = torch.empty((h.shape[0], self.intermediate_size), dtype=self.dtype, device=h.device)
         ws = ctx.workspace if ctx is not None else None

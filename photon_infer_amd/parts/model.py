@@ -148,6 +148,11 @@ class DecoderModel:
             ops.materialize(x, ws)
         return self.head.forward(self.final_norm.forward(x, ctx, rows=ctx.logit_rows), ctx)
 
+    def streamed_weights(self) -> List[torch.Tensor]:
+        """The weight matrices that every decode step reads whole (see ``Part.streamed_weights``)."""
+        parts = [self.embedding, self.final_norm, self.head] + self.blocks
+        return [w for p in parts for w in getattr(p, "streamed_weights", lambda: [])()]
+
     @property
     def graph_safe(self) -> bool:
         """Whether a decode step of this model may be captured as a HIP graph: every part of the

@@ -174,6 +174,28 @@ def test_graph_replayed_decode_equals_eager_steps(tmp_path, dtype, name):
     assert [len(x) for x in graphed] == [14, 17, 20, 9]
 
 
+@pytest.mark.parametrize("name,copies", [("F", 9), ("D", 6), ("E", 2)])
+def test_streaming_copies_of_the_weights_change_no_token(tmp_path, name, copies):
+    """By default the runner keeps a second copy of every matrix that decode steps stream, in the
+    order the kernels load it; a model generates the same tokens with and without (F: all four
+    matrices of both layers and the tied head; D: the down projection's 272 columns and the head's
+    520 rows do not fit the layout's blocks of 16 x 64, the other three per layer do; E, hidden
+    size 160: only the o projection, 160 x 512)."""
+    d = make_model_dir(tmp_path, name, seed=33)
+    vocab = ALL[name][0]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 50 + n) for n in (3, 40, 140)]
+
+    def run(stream_copies):
+        eng = engine(d, name, dtype="bfloat16", stream_copies=stream_copies, chunk_size=64, max_step_tokens=96)
+        out = eng.generate(prompts, max_new_tokens=12, temperature=0.0, ignore_eos=True)
+        return out, eng
+
+    plain, eng0 = run(False)
+    copied, eng1 = run(True)
+    assert eng0.runner.stream_copies == 0 and eng1.runner.stream_copies == copies
+    assert copied == plain
+
+
 @pytest.mark.parametrize("dtype,name", [("float32", "A"), ("bfloat16", "D"), ("bfloat16", "F")])
 def test_a_step_ahead_gives_the_same_tokens(tmp_path, dtype, name):
     """Launching the next decode step before this one's tokens are on the host (they are fed

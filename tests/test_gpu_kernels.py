@@ -265,6 +265,52 @@ def test_gemm_reference_vectors(_ops):
     assert out.cpu().tolist() == [[14.0, 32.0], [32.0, 77.0]]
 
 
+@pytest.mark.parametrize("N,K", [(16, 64), (48, 192), (80, 2048), (1024, 320), (2064, 1088)])
+def test_products_read_a_weight_matrix_or_its_streaming_copy_to_the_same_bits(_ops, N, K):
+    """A workspace may hold a second copy of a weight matrix in the order the weight-streaming
+    kernels load it (16 rows x 64 columns per 2 KB); products of up to 128 tokens then read the
+    copy.  Same arithmetic in the same order, so every bit agrees with the product from the
+    matrix itself: single tokens and the shared-activation kernel, stored, added and left in
+    pieces, the activation in the epilogue, and key ranges merged on the way in."""
+    _ops.use_fast_kernels(True)
+    g = gen(N + K)
+    w = (torch.randn(N, K, generator=g) * 0.1).to(BF16).to(DEV)
+    layout = _ops.stream_layout(w)
+    # the layout itself: lane group lg of a wave holds columns 16 lg + 8 h .. + 7 of row lr in fragment h
+    t = layout.cpu().view(N // 16, K // 64, 2, 4, 16, 8)
+    for rb, kb, h, lg, lr in [(0, 0, 0, 0, 0), (N // 16 - 1, K // 64 - 1, 1, 3, 15), (0, K // 64 - 1, 1, 2, 7)]:
+        k0 = kb * 64 + lg * 16 + h * 8
+        assert torch.equal(t[rb, kb, h, lg, lr], w.cpu()[rb * 16 + lr, k0:k0 + 8])
+    with_copy, without = _ops.KernelWorkspace(DEV), _ops.KernelWorkspace(DEV)
+    assert with_copy.add_stream_copy(w) and not with_copy.add_stream_copy(w[:, :K - 8])
+    for M in (1, 5, 16, 17, 32, 33, 64, 100, 128, 200):
+        a = torch.randn(M, K, generator=g).to(BF16).to(DEV)
+        for c_dtype in (BF16, F32):
+            got, want = torch.empty(M, N, dtype=c_dtype, device=DEV), torch.empty(M, N, dtype=c_dtype, device=DEV)
+            _ops.gemm(got, a, w, ws=with_copy)
+            _ops.gemm(want, a, w, ws=without)
+            assert torch.equal(got, want), f"stored, {M} tokens, {c_dtype}"
+        base = torch.randn(M, N, generator=g).to(DEV)
+        got, want = base.clone(), base.clone()
+        _ops.gemm(got, a, w, accumulate=True, may_defer=True, ws=with_copy)
+        _ops.gemm(want, a, w, accumulate=True, may_defer=True, ws=without)
+        _ops.materialize(got, with_copy)
+        _ops.materialize(want, without)
+        assert torch.equal(got, want), f"added, {M} tokens"
+        close(want, a.double().cpu() @ w.double().cpu().t() + base.double().cpu(), 2e-5, f"against float64, {M} tokens")
+        if N % 32 == 0:
+            got, want = torch.empty(M, N // 2, dtype=BF16, device=DEV), torch.empty(M, N // 2, dtype=BF16, device=DEV)
+            _ops.gemm_swiglu(got, a, w, 16, ws=with_copy)
+            _ops.gemm_swiglu(want, a, w, 16, ws=without)
+            assert torch.equal(got, want), f"activation in the epilogue, {M} tokens"
+    # a slice of the matrix is not the matrix the copy was made of
+    part = torch.empty(4, 16, dtype=F32, device=DEV)
+    _ops.gemm(part, a[:4], w[:16], ws=with_copy)
+    want = torch.empty(4, 16, dtype=F32, device=DEV)
+    _ops.gemm(want, a[:4], w[:16], ws=without)
+    assert torch.equal(part, want)
+
+
 @pytest.mark.parametrize("fast", [False, True])
 def test_gemm_rows_do_not_depend_on_the_batch(_ops, fast):
     """A row's result is the same whatever other rows share the launch."""
@@ -493,6 +539,14 @@ def test_decode_attention_from_projection(_ops, hd, nh, nkv, page, window, rotat
         _ops.gemm(got_b, ranges, w_o, ws=ws)
         assert torch.equal(got_b, want_b)
     assert ws.counts["ranges_merged_by_product"] == 4              # the float32 weights went through the merging kernel
+    # the same from the matrix's copy in the streaming kernels' order
+    w_o = (torch.randn(96, nh * hd, generator=g) * 0.05).to(BF16).to(DEV)
+    copies = _ops.KernelWorkspace(DEV)
+    assert copies.add_stream_copy(w_o)
+    want_x, got_x = torch.empty(R, 96, dtype=F32, device=DEV), torch.empty(R, 96, dtype=F32, device=DEV)
+    _ops.gemm(want_x, ranges, w_o, ws=ws)
+    _ops.gemm(got_x, ranges, w_o, ws=copies)
+    assert torch.equal(got_x, want_x) and copies.counts["ranges_merged_by_product"] == 1
     # and left in pieces for the stream's next norm, as the model's o projection is
     w_o = (torch.randn(96, nh * hd, generator=g) * 0.05).to(BF16).to(DEV)
     x0 = torch.randn(R, 96, generator=g).to(DEV)
