@@ -89,8 +89,9 @@ class KernelWorkspace:
         self.pending: Optional[PendingUpdate] = None
         self.counts: Counter = Counter()
         # weight matrices that have a second copy in the order the weight-streaming kernels read
-        # (steps of up to 128 tokens): address of the matrix -> (copy, rows, columns)
-        self.stream_copies: Dict[int, Tuple[torch.Tensor, int, int]] = {}
+        # (steps of up to 128 tokens): address of the matrix -> (copy, rows, columns, the matrix
+        # itself: while it is kept here, nothing else can come to lie at its address)
+        self.stream_copies: Dict[int, Tuple[torch.Tensor, int, int, torch.Tensor]] = {}
 
     def _buffer(self, name: str, floats: int) -> torch.Tensor:
         buf = getattr(self, name)
@@ -129,7 +130,7 @@ class KernelWorkspace:
         copy = stream_layout(w)
         if copy is None:
             return False
-        self.stream_copies[w.data_ptr()] = (copy, w.shape[0], w.shape[1])
+        self.stream_copies[w.data_ptr()] = (copy, w.shape[0], w.shape[1], w)
         return True
 
     def stream_copy_of(self, w: torch.Tensor, N: int, K: int) -> Optional[torch.Tensor]:
