@@ -2,7 +2,7 @@
 //
 // Reference: include/photon/scheduler/continuous_batch_engine.hpp (ContinuousBatchEngine with
 // add_request(prompt, max_new_tokens) -> id, run_until_complete(), get_result(id)) and
-// include/photon/model/llama_model.hpp.  The names below follow it.
+// include/photon/arch/llama_model.hpp.  The names below follow it.
 //
 // The engine itself (scheduler, step function, kernels' dispatch) lives in the Python package;
 // this library hosts an interpreter inside the calling process and drives that same engine, so

@@ -15,7 +15,8 @@
 //
 // Scores, softmax and both accumulations are float32.  The exponential is taken in base 2:
 // a weight is 2^((score - reference) * scale * log2(e)), one fused multiply-add and v_exp_f32.
-// P is rounded to bfloat16 for the second product; the sum of P is taken before rounding.
+// P is rounded to bfloat16 for the second product; the sum of P is a matrix product too (value
+// rows of ones), so it is the sum of the weights as rounded.
 //
 // The keys and values of a chunk are loaded into registers by attn_load and consumed by
 // attn_compute, so a caller can have the next chunk's loads in flight while it computes.

@@ -11,6 +11,8 @@ import sys
 import time
 from typing import Dict, List, Optional, Sequence
 
+import torch
+
 from ..errors import RequestError
 from ..sampling import Sampler, SamplingParams, uniform_draw
 from .options import EngineOptions
@@ -106,6 +108,13 @@ class ContinuousBatchEngine:
         """Schedule and run one batch; returns the requests known to have finished by the end of
         the call.  With ``lookahead`` a decode step's tokens are read during the next call: the
         step after it is launched first, from what is certain without them."""
+        device = self.runner.device
+        if getattr(device, "type", None) == "cuda" and torch.cuda.current_device() != device.index:
+            with torch.cuda.device(device):      # a process may hold engines on several devices
+                return self._step()
+        return self._step()
+
+    def _step(self) -> List[InferenceRequest]:
         if self._in_flight is not None:
             return self._step_ahead()
         batch = self.scheduler.schedule_next_batch()

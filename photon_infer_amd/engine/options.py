@@ -43,10 +43,14 @@ class EngineOptions:
     max_model_len: Optional[int] = None  # longest sequence; None: the model's max positions
     seed: int = 0
     device: str = "cuda:0"
-    stream_copies: bool = True           # bfloat16 only: keep a second copy of the weight matrices in the order the
-                                         # weight-streaming kernels read them (steps of up to 128 tokens are 2 % faster;
-                                         # costs the matrices' size in device memory again)
+    stream_copies: Optional[bool] = None  # bfloat16 only: keep a second copy of the weight matrices in the order the
+                                         # weight-streaming kernels read them (steps of up to 128 tokens are 2 to 4 % faster;
+                                         # costs the matrices' size in device memory again).  None: if they take at most half
+                                         # of the memory that is free after the weights; True: always, or an error; False: never.
+                                         # The copies are made at load: weights must not be changed afterwards.
     use_graphs: bool = True              # replay HIP graphs for decode-only steps
+    keep_logits: bool = False            # keep a decode step's float32 logits readable until the next decode step
+                                         # (ModelRunner.decode_logits, [requests, vocab]); costs that much memory per graph
     lookahead: bool = True               # schedule a decode step while the one before it still runs (needs use_graphs)
 
     def resolved_dtype(self) -> torch.dtype:

@@ -13,7 +13,9 @@ steps left.  Portions of prompts and single decoded tokens mix freely.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
+import functools
 import gc
+import sys
 from typing import Dict, Hashable, List, Optional, Sequence, Tuple
 
 import numpy as np
@@ -26,6 +28,36 @@ from ..parts import DecoderModel, LayerCache, ModelSpec, StepContext, plan_cache
 from ..registry import build_model_spec, load_config
 from ..weights import load_model_tensors
 from .options import EngineOptions
+
+
+STREAM_COPIES_MAX_SHARE = 0.5     # of the memory that is free after the weights
+
+
+def stream_copies_wanted(copy_bytes: int, free_bytes: int, asked: bool) -> bool:
+    """Whether a runner makes the weights' streaming copies: always when the caller asked for them
+    by name (not fitting is then an ``OutOfMemoryError``); left to itself, when they take at most
+    half of what is free after the weights, so that a model that fills more than a third of the
+    device still loads and keeps a page pool worth having."""
+    if copy_bytes <= 0:
+        return False
+    if asked:
+        if copy_bytes > free_bytes:
+            raise OutOfMemoryError(f"stream_copies=True asks for {copy_bytes / 2**30:.1f} GiB of weight copies; "
+                                   f"{free_bytes / 2**30:.1f} GiB of device memory are free after the weights")
+        return True
+    return copy_bytes <= STREAM_COPIES_MAX_SHARE * free_bytes
+
+
+def _on_own_device(method):
+    """Run a runner's method with the runner's device current: kernels launch on the current
+    device's stream, and a process may hold runners on several devices."""
+    @functools.wraps(method)
+    def wrapped(self, *args, **kwargs):
+        if torch.cuda.current_device() == self.device.index:
+            return method(self, *args, **kwargs)
+        with torch.cuda.device(self.device):
+            return method(self, *args, **kwargs)
+    return wrapped
 
 
 @dataclass
@@ -49,6 +81,14 @@ class ModelRunner:
         self.device = torch.device(self.options.device)
         if self.device.type != "cuda" or not torch.cuda.is_available():
             raise RequestError("the engine runs on a GPU only; no CUDA/HIP device is available")
+        if self.device.index is None:
+            self.device = torch.device("cuda", torch.cuda.current_device())
+        if self.device.index >= torch.cuda.device_count():
+            raise RequestError(f"device {self.options.device}: this process sees {torch.cuda.device_count()} GPU(s)")
+        with torch.cuda.device(self.device):
+            self._load(model_dir, config, tensors)
+
+    def _load(self, model_dir, config, tensors) -> None:
         ops.ensure_loaded(self.dtype)
         self.config = load_config(model_dir) if model_dir is not None else config
         self.spec: ModelSpec = build_model_spec(self.config)
@@ -58,6 +98,12 @@ class ModelRunner:
             from ..weights.loader import check_tensors
             check_tensors({t.name: t for t in self.spec.tensor_specs()}, {n: tuple(t.shape) for n, t in tensors.items()},
                           self.spec.ignorable, "given tensors")
+        if self.dtype == torch.bfloat16:
+            wide = [n for n, t in tensors.items() if t.dtype == torch.float32 and t.dim() >= 2]
+            if wide:
+                print(f"[photon_infer_amd] {len(wide)} weight matrices are stored in 32-bit and stay so ({wide[0]}, ...): "
+                      f"products with them take the float32 kernels, far slower than the bfloat16 ones; "
+                      f"store the folder in bfloat16 to compute in bfloat16", file=sys.stderr, flush=True)
         self.model = DecoderModel(self.spec)
         self.model.load(tensors, self.dtype, self.device)
         del tensors
@@ -68,12 +114,8 @@ class ModelRunner:
         # a second copy of the matrices that every decode step streams, in the order the kernels
         # read them; made before the cache is sized, which takes what memory is left
         self.stream_copies = 0
-        if self.options.stream_copies and self.dtype == torch.bfloat16 and ops.fast_kernels_enabled():
-            seen = set()
-            for w in self.model.streamed_weights():
-                if w is not None and w.data_ptr() not in seen:       # a tied head names the embedding's matrix
-                    seen.add(w.data_ptr())
-                    self.stream_copies += int(self.workspace.add_stream_copy(w))
+        if self.options.stream_copies is not False and self.dtype == torch.bfloat16 and ops.fast_kernels_enabled():
+            self._make_stream_copies()
         self._build_cache()
         # what the mixers want planned on the host per step (equal planners are kept once)
         self.planners = []
@@ -86,6 +128,37 @@ class ModelRunner:
         self.graph_safe = self.model.graph_safe
         self._graphs: Dict[Tuple[int, int], "_DecodeGraph"] = {}
 
+    # ------------------------------------------------------------------ the weights' streaming copies
+    def _free_device_bytes(self) -> int:
+        free, _total = torch.cuda.mem_get_info(self.device)
+        return free + torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device)   # torch's own spare blocks
+
+    def _make_stream_copies(self) -> None:
+        """Copy the streamed matrices if that leaves room for a useful page pool
+        (``stream_copies_wanted``); running out of memory on the way drops them all again.  The
+        model runs without them, a little slower; only a caller who asked for them by
+        ``stream_copies=True`` gets an error instead."""
+        seen, mats = set(), []
+        for w in self.model.streamed_weights():
+            if w is not None and w.data_ptr() not in seen and ops.stream_layout_takes(w):   # a tied head names the embedding's matrix
+                seen.add(w.data_ptr())
+                mats.append(w)
+        need = sum(w.numel() * w.element_size() for w in mats)
+        asked = self.options.stream_copies is True
+        if not stream_copies_wanted(need, self._free_device_bytes(), asked):
+            return
+        try:
+            for w in mats:
+                self.stream_copies += int(self.workspace.add_stream_copy(w))
+        except torch.OutOfMemoryError:
+            self.workspace.drop_stream_copies()
+            self.stream_copies = 0
+            if asked:
+                raise OutOfMemoryError(f"stream_copies=True: the weights' streaming copies ({need / 2**30:.1f} GiB) "
+                                       f"do not fit the device") from None
+            print(f"[photon_infer_amd] no room for the weights' streaming copies ({need / 2**30:.1f} GiB): running without them",
+                  file=sys.stderr, flush=True)
+
     # ------------------------------------------------------------------ cache set-up
     def _build_cache(self) -> None:
         o = self.options
@@ -97,8 +170,7 @@ class ModelRunner:
         # bytes of keys and values that one page holds over all layers that own pages
         itemsize = torch.empty((), dtype=self.dtype).element_size()
         page_bytes = sum(2 * nkv * hd * self.page_size * itemsize for g in self.plan.groups for nkv, hd in g.kv_shapes)
-        free, _total = torch.cuda.mem_get_info(self.device)
-        free += torch.cuda.memory_reserved(self.device) - torch.cuda.memory_allocated(self.device)   # torch's own spare blocks
+        free = self._free_device_bytes()
         if o.num_blocks is not None or o.max_cache_tokens is not None:
             num_pages = int(o.num_blocks) if o.num_blocks is not None else max(1, -(-int(o.max_cache_tokens) // self.page_size))
             if num_pages <= 0:
@@ -180,6 +252,9 @@ class ModelRunner:
             for w in e.want:
                 if not 0 <= int(w) < n:
                     raise RequestError(f"request {e.rid!r}: wanted row {w} is outside its {n} tokens")
+            if len(e.want) > 1 and len(set(int(w) for w in e.want)) != len(e.want):
+                # the final norm folds a pending update into each wanted row, one block per row
+                raise RequestError(f"request {e.rid!r}: a row is wanted twice ({list(e.want)})")
             if self.cache.length(e.rid) + n > self.max_model_len:
                 raise RequestError(
                     f"request {e.rid!r} would reach {self.cache.length(e.rid) + n} tokens; the limit is {self.max_model_len}")
@@ -234,6 +309,7 @@ class ModelRunner:
         self.cache.reserve_step(slots, [len(e.tokens) for e in entries])
         return slots
 
+    @_on_own_device
     @torch.no_grad()
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Run one batch.  Returns float32 logits [wanted rows, vocab] on the device, in
@@ -249,6 +325,7 @@ class ModelRunner:
         return logits
 
     graphs_captured = 0
+    decode_logits: Optional[torch.Tensor] = None     # with options.keep_logits: the last decode step's logits [R, vocab]
 
     # what a caller that reads a step's tokens later needs: an event to record behind its copy
     # and page-locked memory to copy into
@@ -268,6 +345,7 @@ class ModelRunner:
             self._graph_pool = torch.cuda.graph_pool_handle()
         return self._graph_pool
 
+    @_on_own_device
     @torch.no_grad()
     def decode_step(self, entries: Sequence[StepEntry], temperatures: Sequence[float], uniforms: Sequence[float],
                     feed: Optional[Tuple[torch.Tensor, Sequence[int]]] = None) -> torch.Tensor:
@@ -299,6 +377,7 @@ class ModelRunner:
         if graph is None:
             graph = self._graphs[(len(entries), bucket)] = _DecodeGraph(self, len(entries), bucket)
         out = graph.run(entries, slots, lengths, temperatures, uniforms, feed)
+        self.decode_logits = graph.logits
         self.cache.commit_step(slots, [1] * len(slots))
         return out
 
@@ -314,6 +393,7 @@ class ModelRunner:
             rows = torch.tensor(list(feed[1]), dtype=torch.int32).to(self.device)
             torch.index_select(feed[0], 0, rows, out=ctx.token_ids)
         logits = self.model.forward(ctx, self.layer_caches)
+        self.decode_logits = logits if self.options.keep_logits else None
         params = torch.from_numpy(np.asarray([list(temperatures), list(uniforms)], np.float32)).to(self.device)
         out = torch.empty(R, dtype=torch.int32, device=self.device)   # a buffer of its own: the step before may still be unread
         ops.sample(out, logits, params[0], params[1], ws=self.workspace)
@@ -372,6 +452,7 @@ class _DecodeGraph:
         self.temps = d["temps"].view(torch.float32)
         self.uniforms = d["uniforms"].view(torch.float32)
         self.sampled = torch.zeros(R, dtype=torch.int32, device=runner.device)
+        self.logits: Optional[torch.Tensor] = None
         self.graph: Optional[torch.cuda.CUDAGraph] = None
 
     def _fill(self, entries, slots, lengths, temperatures, uniforms, feed) -> None:
@@ -399,6 +480,9 @@ class _DecodeGraph:
     def _body(self) -> None:
         logits = self.runner.model.forward(self.ctx, self.runner.layer_caches)
         ops.sample(self.sampled, logits, self.temps, self.uniforms, ws=self.runner.workspace)
+        # kept alive, the logits stay where every replay writes them (and the pool cannot give
+        # their memory to another graph); otherwise a graph holds nothing between replays
+        self.logits = logits if self.runner.options.keep_logits else None
 
     def run(self, entries, slots, lengths, temperatures, uniforms, feed=None) -> torch.Tensor:
         self._fill(entries, slots, lengths, temperatures, uniforms, feed)
@@ -409,8 +493,10 @@ class _DecodeGraph:
             # work, and the capture that follows only records.  Every later graph is captured
             # straight away and replayed for its first step.
             eager_first = not runner.graphs_captured
+            first_logits = None
             if eager_first:
                 self._body()
+                first_logits = self.logits
                 torch.cuda.synchronize()
             graph = torch.cuda.CUDAGraph()
             # no garbage collection while the stream is capturing: a collected tensor of some
@@ -439,6 +525,8 @@ class _DecodeGraph:
             runner.graphs_captured += 1
             if not eager_first:
                 graph.replay()
+            elif first_logits is not None:
+                self.logits.copy_(first_logits)      # the capture recorded only: this step's logits are the eager run's
         else:
             self.graph.replay()
         return self.sampled

@@ -17,7 +17,7 @@ import torch
 
 from ..errors import KernelError
 from . import _lib
-from .workspace import KernelWorkspace, KeyRanges, Partials, stream_layout
+from .workspace import KernelWorkspace, KeyRanges, Partials, stream_layout, stream_layout_takes
 
 PI_F32, PI_BF16 = 0, 1
 MAX_HEAD_DIM = 256

@@ -3,7 +3,7 @@ from __future__ import annotations
 
 import ctypes
 from ctypes import c_float, c_int, c_long, c_void_p
-from typing import Dict, Optional
+from typing import Dict
 
 import torch
 
@@ -43,19 +43,17 @@ _LIBS: Dict[str, ctypes.CDLL] = {}
 
 
 _RAW_STREAM = getattr(torch._C, "_cuda_getCurrentRawStream", None)
-_DEVICE_INDEX: Optional[int] = None
+_CURRENT_DEVICE = getattr(torch._C, "_cuda_getDevice", None)
 
 
 def current_stream() -> int:
-    """The current HIP stream's handle.  Asked for at every kernel launch (a step of a few
-    hundred launches), so by the shortest way torch offers: its Python-level
-    ``current_stream()`` costs as much as the launch itself."""
-    global _DEVICE_INDEX
-    if _RAW_STREAM is None:
+    """The handle of torch's current HIP stream on the current device (whoever launches kernels
+    for tensors of another device makes that device current first; ``ModelRunner`` does).  Asked
+    for at every kernel launch (a step of a few hundred launches), so by the shortest way torch
+    offers: its Python-level ``current_stream()`` costs as much as the launch itself."""
+    if _RAW_STREAM is None or _CURRENT_DEVICE is None:
         return torch.cuda.current_stream().cuda_stream
-    if _DEVICE_INDEX is None:
-        _DEVICE_INDEX = torch.cuda.current_device()      # one process, one GPU
-    return _RAW_STREAM(_DEVICE_INDEX)
+    return _RAW_STREAM(_CURRENT_DEVICE())
 
 
 def load(module: str) -> ctypes.CDLL:

@@ -5,8 +5,8 @@ ones its kernels take, in which case the caller uses the general kernel.
 
 Which kernel takes what:
   * matrix products: K and the row strides multiples of 8, 16-byte aligned operands;
-    up to 64 rows go to the weight-streaming kernel (k split over blocks where the output
-    is narrow), more rows to the 128 x 128 tile kernel;
+    up to 128 rows go to the weight-streaming kernels (k split over blocks where the output
+    is narrow), more rows to the tile kernels;
   * attention: pages of a multiple of 16 tokens; a batch of single tokens with at most 16 heads
     per kv head goes to the key-split decode kernel (head_dim a multiple of 16 up to 256; for
     64 and 128 straight from the q|k|v projection), any other batch to the tile kernel

@@ -61,16 +61,20 @@ class PendingUpdate:
         return t is x or (t.data_ptr() == x.data_ptr() and t.shape == x.shape and t.stride() == x.stride())
 
 
+def stream_layout_takes(w: torch.Tensor) -> bool:
+    """Whether ``stream_layout`` has a form for ``w``."""
+    return (w.dim() == 2 and w.dtype == torch.bfloat16 and w.is_contiguous() and w.shape[0] > 0 and w.shape[0] % 16 == 0
+            and w.shape[1] > 0 and w.shape[1] % 64 == 0)
+
+
 def stream_layout(w: torch.Tensor) -> Optional[torch.Tensor]:
     """The bfloat16 matrix ``w`` [N, K] (N a multiple of 16, K of 64, rows contiguous) as
     [N / 16][K / 64][2][4][16][8]: for every 16 rows and 64 columns, the 1 KB that a wave of the
     weight-streaming kernels loads with one instruction lies in a row (lane group g of a wave
     holds columns 16 g + 8 h .. + 7 of its row in its fragment h).  None for other matrices."""
-    if w.dim() != 2 or w.dtype != torch.bfloat16 or not w.is_contiguous():
+    if not stream_layout_takes(w):
         return None
     N, K = w.shape
-    if N == 0 or N % 16 or K == 0 or K % 64:
-        return None
     tiles = w.view(N // 16, 16, K // 64, 4, 2, 8)          # [row block, row, k block, lane group, fragment, 8 columns]
     return tiles.permute(0, 2, 4, 3, 1, 5).contiguous().view(N, K)
 
@@ -132,6 +136,12 @@ class KernelWorkspace:
             return False
         self.stream_copies[w.data_ptr()] = (copy, w.shape[0], w.shape[1], w)
         return True
+
+    def drop_stream_copies(self) -> None:
+        """Forget every copy (their memory goes back to the allocator); products read the matrices
+        themselves again.  For a caller that changes a weight matrix after load: a copy is made
+        once and never refreshed."""
+        self.stream_copies.clear()
 
     def stream_copy_of(self, w: torch.Tensor, N: int, K: int) -> Optional[torch.Tensor]:
         entry = self.stream_copies.get(w.data_ptr())

@@ -232,3 +232,23 @@ def test_engine_refuses_tokens_outside_the_vocabulary():
     eng = ContinuousBatchEngine(None, runner=StandInRunner(opts, 64))
     with pytest.raises(RequestError):
         eng.add_request([1, VOCAB], 4)
+
+
+def test_the_decision_to_copy_the_weights_for_streaming():
+    """Left to itself a runner makes the copies only when they take at most half of the memory that
+    is free after the weights; asked for by name they are made whenever they fit, and refused with
+    the engine's own error when they do not."""
+    from photon_infer_amd.engine.step import stream_copies_wanted
+    from photon_infer_amd.errors import ErrorCode, OutOfMemoryError
+
+    GiB = 1 << 30
+    assert stream_copies_wanted(2 * GiB, 280 * GiB, asked=False)            # 1B sizes on an empty device
+    assert stream_copies_wanted(16 * GiB, 250 * GiB, asked=False)           # 8B sizes
+    assert not stream_copies_wanted(130 * GiB, 140 * GiB, asked=False)      # weights take half the device: none
+    assert not stream_copies_wanted(71 * GiB, 140 * GiB, asked=False)
+    assert stream_copies_wanted(70 * GiB, 140 * GiB, asked=False)
+    assert not stream_copies_wanted(0, 140 * GiB, asked=False) and not stream_copies_wanted(0, 140 * GiB, asked=True)
+    assert stream_copies_wanted(130 * GiB, 140 * GiB, asked=True)           # asked for: made while they fit
+    with pytest.raises(OutOfMemoryError, match="stream_copies=True") as err:
+        stream_copies_wanted(150 * GiB, 140 * GiB, asked=True)
+    assert err.value.code == ErrorCode.OUT_OF_MEMORY

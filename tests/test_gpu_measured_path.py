@@ -1,0 +1,181 @@
+"""The paths that the benchmark times, under a comparison.
+
+Decode steps replayed from graphs whose attention is cut into several key ranges (contexts past
+128, 256 and 512 tokens, the ranges merged by the o projection), the switch from one length
+bucket's graph to the next, the step launched ahead - against eager steps and against the plain
+implementation; and the chain of kernels that runs at the benchmark's own layer sizes (hidden
+2,048, intermediate 8,192, 32 heads on 8 of 64, a vocabulary of 128,256), two layers of it,
+against the plain implementation: a 2,048-token prompt whole, then decode steps of batch 8.
+"""
+import pytest
+import torch
+
+import plain_llama as P
+import plain_wide as PW
+from tiny_models import ALL, make_model_dir, random_tokens
+
+pytestmark = pytest.mark.gpu
+
+# batch size -> (prompt lengths, new tokens): contexts cross 128, 256 and 512 while decoding
+CASES = {
+    1: ([120], [140]),
+    3: ([100, 250, 490], [40, 60, 80]),
+    8: ([100, 118, 230, 250, 300, 470, 490, 60], [60, 40, 50, 80, 40, 60, 45, 70]),
+}
+
+
+@pytest.fixture(scope="module")
+def model_dirs(tmp_path_factory):
+    root = tmp_path_factory.mktemp("models")
+    return {name: make_model_dir(root, name, seed=51) for name in ("D", "F")}
+
+
+def engine(model_dir, name, **kw):
+    from photon_infer_amd import ContinuousBatchEngine
+    opts = dict(dtype="bfloat16", block_size=16, num_blocks=256, max_batch=8, max_model_len=1024, chunk_size=128,
+                max_step_tokens=256)
+    opts.update(kw)
+    return ContinuousBatchEngine(model_dir, **opts)
+
+
+def generate(eng, prompts, new_tokens, temperatures):
+    ids = [eng.add_request(p, n, temperature=t, seed=11 + i, ignore_eos=True)
+           for i, (p, n, t) in enumerate(zip(prompts, new_tokens, temperatures))]
+    eng.run_until_complete()
+    assert eng.runner.cache.num_live == 0
+    eng.runner.cache.check_invariants()
+    return [eng.get_result(i) for i in ids]
+
+
+@pytest.mark.parametrize("batch", [1, 3, 8])
+@pytest.mark.parametrize("name", ["D", "F"])
+def test_graphs_over_several_key_ranges_equal_eager_steps(model_dirs, name, batch):
+    """Greedy and sampled requests whose contexts pass 128, 256 and 512 tokens while they decode:
+    every decode step's attention is cut into key ranges that the o projection merges, one graph
+    per (batch size, length bucket) is captured and left behind, and the tokens are those of the
+    same steps launched kernel by kernel; launching a step ahead changes nothing either (every
+    request is there from the start and ends by its length, so the batches are the same)."""
+    lengths, new_tokens = CASES[batch]
+    vocab = ALL[name][0]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 300 + n) for n in lengths]
+    temps = [0.0 if i % 2 == 0 else 0.8 for i in range(batch)]
+
+    def run(use_graphs, lookahead):
+        eng = engine(model_dirs[name], name, use_graphs=use_graphs, lookahead=lookahead)
+        return generate(eng, prompts, new_tokens, temps), eng
+
+    eager, e0 = run(False, False)
+    graphed, e1 = run(True, False)
+    ahead, e2 = run(True, True)
+    assert [len(x) for x in eager] == new_tokens
+    assert not e0.runner._graphs and len(e1.runner._graphs) >= 3, sorted(e1.runner._graphs)
+    assert len({bucket for _, bucket in e1.runner._graphs}) >= 2          # more than one length bucket was decoded in
+    assert all(g.graph is not None for g in e1.runner._graphs.values())
+    for e in (e0, e1, e2):
+        assert e.runner.workspace.counts["ranges_merged_by_product"] > 0, e.runner.workspace.counts
+    assert graphed == eager
+    assert ahead == eager
+
+
+@pytest.mark.parametrize("name", ["D", "F"])
+def test_greedy_decoding_past_several_buckets_follows_the_plain_arg_max(model_dirs, name):
+    """The same requests, greedy, through the default engine (graphs, a step ahead): every token
+    is the plain implementation's arg max, or within the slack that bfloat16 rounding leaves
+    between two candidates."""
+    lengths, new_tokens = CASES[3]
+    vocab = ALL[name][0]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 300 + n) for n in lengths]
+    eng = engine(model_dirs[name], name)
+    outs = generate(eng, prompts, new_tokens, [0.0] * 3)
+    assert len(eng.runner._graphs) >= 3 and eng.runner.workspace.counts["ranges_merged_by_product"] > 0
+    cfg, W = P.read_model_folder(model_dirs[name])
+    for p, out in zip(prompts, outs):
+        seq = list(p) + list(out)
+        rows = list(range(len(p) - 1, len(seq) - 1))                     # the rows that chose the new tokens
+        ref = PW.llama_forward(cfg, W, seq, rows, device="cuda").cpu()
+        emu = PW.llama_forward(cfg, W, seq, rows, act_round=P.bf16_round, device="cuda").cpu()
+        slack = 3.0 * (emu - ref).abs().max().item()
+        for k, tok in enumerate(out):
+            assert ref[k, tok].item() >= ref[k].max().item() - 2 * slack, (len(p), k, tok)
+
+
+# ------------------------------------------------------------------ the benchmark's layer sizes
+BENCH_SIZES = dict(
+    architectures=["LlamaForCausalLM"], hidden_size=2048, intermediate_size=8192, num_hidden_layers=2,
+    num_attention_heads=32, num_key_value_heads=8, head_dim=64, vocab_size=128256,
+    max_position_embeddings=131072, rms_norm_eps=1e-5, rope_theta=500000.0,
+    rope_scaling=dict(rope_type="llama3", factor=32.0, low_freq_factor=1.0, high_freq_factor=4.0,
+                      original_max_position_embeddings=8192),
+    tie_word_embeddings=True,
+)
+
+
+def test_two_layers_at_the_benchmark_sizes_against_the_plain_implementation(monkeypatch):
+    """What ``bench.py`` times, compared: a 2,048-token prompt in one step (the large-tile product
+    fed k in four pieces, the o projection in pieces, prompt attention over 16 rounds), then 16
+    decode steps of batch 8 through ``decode_step`` (graphs of the 4,096 bucket: eight key ranges
+    merged by the o projection, every product streamed in eight pieces, the output head over
+    128,256 rows, the two-kernel sampler), logits of the prompts' last rows and of every decode
+    row against the plain implementation."""
+    from photon_infer_amd.config import LlamaConfig
+    from photon_infer_amd.engine import EngineOptions, ModelRunner, StepEntry
+    from photon_infer_amd.ops import fast
+    from photon_infer_amd.registry import build_model_spec
+
+    cfg = LlamaConfig.from_dict(BENCH_SIZES)
+    spec = build_model_spec(cfg)
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    tensors = {}
+    for s in spec.tensor_specs():
+        if s.role == "norm":
+            t = torch.rand(s.shape, generator=gen, device="cuda") + 0.5
+        else:
+            t = torch.randn(s.shape, generator=gen, device="cuda") * 0.02
+        tensors[s.name] = t.to(torch.bfloat16)
+    plain_weights = dict(tensors)
+
+    calls = {"tile": [], "skinny": []}
+    tile_splits, skinny_splits = fast._tile_splits, fast._skinny_splits
+    monkeypatch.setattr(fast, "_tile_splits", lambda M, N, K: calls["tile"].append((M, N, K, tile_splits(M, N, K))) or calls["tile"][-1][3])
+    monkeypatch.setattr(fast, "_skinny_splits", lambda M, N, K: calls["skinny"].append((M, N, K, skinny_splits(M, N, K))) or calls["skinny"][-1][3])
+
+    lengths = [2048, 1500, 900, 400, 130, 2000, 64, 1024]
+    steps = 16
+    runner = ModelRunner(None, EngineOptions(max_batch=8, max_cache_tokens=8 * (2048 + 64), max_model_len=4096, keep_logits=True),
+                         config=cfg, tensors=tensors)
+    assert runner.stream_copies == 9 and runner.graph_safe
+    prompts = [random_tokens(n, cfg.vocab_size, 500 + n) for n in lengths]
+    rids = [f"r{i}" for i in range(8)]
+    got = [[] for _ in rids]                                  # per request: logits rows, the prompt's last first
+    seqs = [list(p) for p in prompts]
+    for i, (rid, p) in enumerate(zip(rids, prompts)):
+        runner.admit(rid)
+        logits = runner.step([StepEntry(rid, p, [len(p) - 1])])
+        got[i].append(logits[0].cpu())
+        seqs[i].append(int(logits[0].argmax()))
+    assert (2048, 2048, 8192, 4) in calls["tile"], calls["tile"]          # the down projection of the whole prompt
+    for _ in range(steps):
+        ids = runner.decode_step([StepEntry(rid, [seq[-1]], [0]) for rid, seq in zip(rids, seqs)], [0.0] * 8, [0.0] * 8)
+        logits = runner.decode_logits.cpu()
+        for i, tok in enumerate(ids.tolist()):
+            got[i].append(logits[i].clone())
+            assert tok == int(logits[i].argmax())             # the graph's sampler chose this row's first maximum
+            seqs[i].append(tok)
+    assert list(runner._graphs) == [(8, 4096)]
+    counts = runner.workspace.counts
+    assert counts["ranges_merged_by_product"] >= 2 * steps and counts["qkv_pieces"] > 0 and counts["added_by_norm"] > 0, counts
+    assert (8, 2048, 2048, 8) in calls["skinny"] and (8, 2048, 8192, 8) in calls["skinny"], set(calls["skinny"])
+    for rid in rids:
+        runner.release(rid)
+
+    raw = cfg.to_dict()
+    for i, p in enumerate(prompts):
+        seq = seqs[i][:-1]                                    # the last token was chosen and never fed
+        rows = list(range(len(p) - 1, len(seq)))
+        assert len(rows) == steps + 1 == len(got[i])
+        ref = PW.llama_forward(raw, plain_weights, seq, rows, device="cuda").cpu()
+        emu = PW.llama_forward(raw, plain_weights, seq, rows, act_round=P.bf16_round, device="cuda").cpu()
+        tol = 3.0 * (emu - ref).abs().max().item()
+        err = max((g - r).abs().max().item() for g, r in zip(got[i], ref))
+        assert err <= tol, (i, len(p), err, tol)
+        assert tol < 0.2 * ref.abs().max().item()             # the yardstick itself is tight

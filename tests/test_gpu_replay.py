@@ -246,6 +246,8 @@ def test_step_preconditions(model_dirs):
         runner.step([StepEntry("x", [1]), StepEntry("x", [2])])
     with pytest.raises(RequestError, match="wanted row"):
         runner.step([StepEntry("x", [1, 2], [2])])
+    with pytest.raises(RequestError, match="wanted twice"):
+        runner.step([StepEntry("x", [1, 2], [0, 1, 0])])
     runner.admit("y")
     with pytest.raises(OutOfPagesError):
         runner.step([StepEntry("x", [1] * 40), StepEntry("y", [1] * 40)])

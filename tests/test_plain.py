@@ -262,3 +262,29 @@ def test_float64_agrees_with_float32():
     a = P.llama_forward(cfg, W, toks)
     b = P.llama_forward(cfg, W, toks, dtype=torch.float64)
     assert (a.double() - b).abs().max() < 5e-5 * b.abs().max().clamp(min=1)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_the_whole_tensor_form_equals_the_loops(name):
+    """``plain_wide`` (the same formulas over whole tensors, used where sequences are thousands of
+    tokens long) against ``plain_llama``: with and without the bfloat16 rounding points, with a
+    window, for all rows and for chosen rows, interleaved pairs too."""
+    import plain_wide as PW
+    from tiny_models import ALL
+
+    raw, init = ALL[name]
+    cfg, W = _tiny(raw, seed=3, std=init["std"])
+    toks = torch.randint(0, raw["vocab_size"], (37,), generator=torch.Generator().manual_seed(8)).tolist()
+    ref = P.llama_forward(cfg, W, toks)
+    tol = 2e-5 * max(1.0, ref.abs().max().item())
+    assert (PW.llama_forward(cfg, W, toks) - ref).abs().max() < tol
+    assert (PW.llama_forward(cfg, W, toks, rows=[36, 0, 17]) - ref[[36, 0, 17]]).abs().max() < tol
+    emu = P.llama_forward(cfg, W, toks, act_round=P.bf16_round)
+    wide = PW.llama_forward(cfg, W, toks, act_round=P.bf16_round)
+    # rounding points make the two forms differ where a value sits on a rounding boundary; the
+    # deviation stays far below what the rounding itself does to the logits
+    assert (wide - emu).abs().max() < 0.25 * (emu - ref).abs().max()
+    win = P.llama_forward(cfg, W, toks, window=5)
+    assert (PW.llama_forward(cfg, W, toks, window=5) - win).abs().max() < tol and (win - ref).abs().max() > 10 * tol
+    inter = dict(cfg, rope_interleaved=True)
+    assert (PW.llama_forward(inter, W, toks) - P.llama_forward(inter, W, toks)).abs().max() < tol
