@@ -163,7 +163,8 @@ def test_two_layers_at_the_benchmark_sizes_against_the_plain_implementation(monk
             seqs[i].append(tok)
     assert list(runner._graphs) == [(8, 4096)]
     counts = runner.workspace.counts
-    assert counts["ranges_merged_by_product"] >= 2 * steps and counts["qkv_pieces"] > 0 and counts["added_by_norm"] > 0, counts
+    # (counted where Python launches: the eager first step and the capture, not the replays)
+    assert counts["ranges_merged_by_product"] >= 2 and counts["qkv_pieces"] > 0 and counts["added_by_norm"] > 0, counts
     assert (8, 2048, 2048, 8) in calls["skinny"] and (8, 2048, 8192, 8) in calls["skinny"], set(calls["skinny"])
     for rid in rids:
         runner.release(rid)
