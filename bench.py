@@ -1,7 +1,8 @@
 #!/usr/bin/python3
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode1b|serve3b|mixed8b]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode1b|long1b|serve3b|mixed8b]
+                    [--batch 8,1,64] [--context 4096] [--dtype bf16|fp32]
 
 Every workload prints ONE JSON line.  The default, ``decode1b`` (Llama 3.2 1B layer sizes):  ``value`` is decoded tokens per second at batch 8 with the context
 length of the benchmark configuration (every request's cache holds that many tokens when
@@ -14,6 +15,17 @@ decode step has to read / its time, against 8 TB/s) and ``points`` (batch 1 and 
 ``points`` also holds ``engine_b8``: decoded tokens per second of the same batch through
 ``ContinuousBatchEngine`` (scheduler, request objects, sampling, the step ahead), measured over its
 decode phase.
+
+``--batch a,b,c``: the first is the headline's batch, the others become ``points.decode_b<b>``;
+``--context N``: the context length the decode steps end at.  ``--dtype fp32`` runs the same
+workload on the float32 path (true 32-bit kernels; the caches are then filled with random
+numbers instead of running 4,096-token prompts through them).
+
+``--workload long1b`` (the same model): decode steps at further sizes over caches of random
+numbers - batch 8 at a context of 32,768, one request at 131,000, batch 64 at 8,192 - and one
+512-token portion of a prompt at the end of a context of 16,384, each with the bytes it has to
+read or the flops it does against the peaks.  After demo/compare_batching_methods.cpp:251-309 of
+the reference, which prints a throughput per workload.
 
 ``--workload serve3b`` (Llama 3.2 3B layer sizes): continuous batching of 64 requests, prompts of
 128 to 2,048 tokens, 64 to 512 new tokens each, 16 there at the start and 4 more every 8 steps,
@@ -286,6 +298,76 @@ def workload_serve3b(args) -> int:
     return 0
 
 
+def time_late_portion(runner, portion, context, reps, seed=4):
+    """Seconds per step of one ``portion``-token piece of a prompt that ends at ``context``, over
+    a cache of random numbers (the pages before it reserved, not computed)."""
+    import torch
+
+    from photon_infer_amd.engine import StepEntry
+
+    g = torch.Generator().manual_seed(seed)
+    toks = torch.randint(0, runner.spec.vocab_size, (portion,), generator=g).tolist()
+
+    def once(i):
+        rid = f"late{i}"
+        runner.admit(rid)
+        runner.cache.reserve(rid, context - portion)
+        runner.cache.commit(rid, context - portion)
+        runner.step([StepEntry(rid, toks, [portion - 1])])
+        runner.release(rid)
+
+    once(-1)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(reps):
+        once(i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / reps
+
+
+def workload_long1b(args) -> int:
+    """Decode steps and a late prompt portion at long contexts, Llama 3.2 1B layer sizes (see the
+    module text).  One runner whose pool holds the largest case."""
+    layers = args.layers or MODEL["num_hidden_layers"]
+    cases = [(8, 32768), (1, 131000), (64, 8192)]
+    portion, portion_ctx = 512, 16384
+    pool = max(b * (c + 64) for b, c in cases)
+    runner, cfg = make_runner(MODEL, layers, args.dtype, 64, pool, max_model_len=131072)
+    elem = 2 if args.dtype == "bf16" else 4
+    wbytes, kvb = weight_bytes(runner), kv_bytes_per_token(cfg, layers, elem)
+    points = {}
+    for b, c in cases:
+        sec, mean_ctx = time_decode(runner, b, args.steps, args.warmup, c, synthetic_cache=True)
+        gbs = (wbytes + b * mean_ctx * kvb) / sec / 1e9
+        points[f"decode_b{b}_ctx{c}"] = {"ms_per_step": round(sec * 1e3, 4), "tokens_per_s": round(b / sec, 1),
+                                         "GB_per_s": round(gbs, 1), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4)}
+    psec = time_late_portion(runner, portion, portion_ctx, max(2, min(8, args.steps)))
+    per_layer = cfg.hidden_size * (cfg.q_size + 2 * cfg.kv_size) + cfg.q_size * cfg.hidden_size + 3 * cfg.hidden_size * cfg.intermediate_size
+    flops = 2.0 * portion * per_layer * layers + 2.0 * cfg.hidden_size * cfg.vocab_size \
+        + layers * 4.0 * cfg.num_attention_heads * cfg.head_dim * portion * (portion_ctx - portion / 2.0)
+    points[f"portion{portion}_ctx{portion_ctx}"] = {"ms": round(psec * 1e3, 3), "tokens_per_s": round(portion / psec, 1),
+                                                    "frac_of_flops_peak": round(flops / psec / PEAK_FLOPS[args.dtype], 4)}
+    head = points["decode_b8_ctx32768"]
+    line = {
+        "metric": "decode tok/s at batch 8, context 32768 (Llama 3.2 1B layer sizes, random weights, random cache contents)",
+        "value": head["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), random cache contents, uniform random token ids",
+        "config": {
+            "model": "llama-3.2-1b-sizes", "layers": layers, "layers_of_model": MODEL["num_hidden_layers"],
+            "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
+            "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+            "tied_embeddings": cfg.tie_word_embeddings, "global_batch": 8, "seq_len": 32768, "kv_block": BLOCK_SIZE,
+            "parallelism": "single-gpu", "weight_bytes": wbytes, "kv_bytes_per_token": kvb,
+        },
+        "roofline": {"bound": "hbm", "achieved": head["GB_per_s"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": head["frac_of_hbm_peak"]},
+        "points": points,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
 def workload_mixed8b(args) -> int:
     """Mixed steps at Llama 3.1 8B layer sizes (see the module text)."""
     import torch
@@ -359,8 +441,10 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
     ap.add_argument("--warmup", type=int, default=8)
-    ap.add_argument("--batch", type=int, default=8)
-    ap.add_argument("--workload", choices=["decode1b", "serve3b", "mixed8b"], default="decode1b")
+    ap.add_argument("--batch", default="8,1,64",
+                    help="batch sizes of the decode steps: the first is the headline's, the others become points")
+    ap.add_argument("--context", type=int, default=CONTEXT, help="context length that the decode steps end at")
+    ap.add_argument("--workload", choices=["decode1b", "long1b", "serve3b", "mixed8b"], default="decode1b")
     ap.add_argument("--layers", type=int, default=None,
                     help="fewer layers than the model has, if memory or time needs it (both numbers are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "fp32"])
@@ -377,14 +461,27 @@ def main() -> int:
     if not torch.cuda.is_available():
         print("bench.py: no GPU available", file=sys.stderr)
         return 1
+    batches = [int(b) for b in str(args.batch).split(",") if b]
+    if not batches or min(batches) < 1:
+        print(f"bench.py: --batch {args.batch} names no batch size", file=sys.stderr)
+        return 1
+    args.batch, more_batches = batches[0], batches[1:]
+    context = args.context
+    if context <= args.steps + args.warmup:
+        print(f"bench.py: --context {context} is shorter than the {args.steps + args.warmup} steps to run", file=sys.stderr)
+        return 1
+    if args.workload == "long1b":
+        return workload_long1b(args)
     if args.workload == "serve3b":
         return workload_serve3b(args)
     if args.workload == "mixed8b":
         return workload_mixed8b(args)
     args.layers = args.layers or MODEL["num_hidden_layers"]
     elem = 2 if args.dtype == "bf16" else 4
-    big = 1 if (args.no_points or args.only) else 64
-    runner, cfg = make_runner(MODEL, args.layers, args.dtype, max(big, args.batch), (max(big, args.batch)) * (CONTEXT + 64))
+    big = args.batch if (args.no_points or args.only) else max(batches)
+    synthetic = args.dtype == "fp32"      # the float32 kernels would spend minutes on the prompts that fill the caches
+    runner, cfg = make_runner(MODEL, args.layers, args.dtype, big, max(big * (context + 64), PREFILL_TOKENS + 64),
+                              max_model_len=max(context, PREFILL_TOKENS) + 64)
     wbytes = weight_bytes(runner)
     kvb = kv_bytes_per_token(cfg, args.layers, elem)
     if args.only == "prefill":
@@ -392,26 +489,27 @@ def main() -> int:
         print(json.dumps({"only": "prefill", "tokens": PREFILL_TOKENS, "ms": round(psec * 1e3, 3)}), flush=True)
         return 0
     if args.only == "decode":
-        sec, _ = time_decode(runner, args.batch, args.steps, args.warmup, CONTEXT, synthetic_cache=True)
+        sec, _ = time_decode(runner, args.batch, args.steps, args.warmup, context, synthetic_cache=True)
         print(json.dumps({"only": "decode", "batch": args.batch, "ms_per_step": round(sec * 1e3, 4),
                           "cache": "random numbers, no prompt was run"}), flush=True)
         return 0
 
-    sec, mean_ctx = time_decode(runner, args.batch, args.steps, args.warmup, CONTEXT)
+    sec, mean_ctx = time_decode(runner, args.batch, args.steps, args.warmup, context, synthetic_cache=synthetic)
     value = args.batch / sec
     step_bytes = wbytes + args.batch * mean_ctx * kvb
     achieved = step_bytes / sec / 1e9
     line = {
-        "metric": "decode tok/s at batch 8, context 4096 (Llama 3.2 1B layer sizes, random weights)",
+        "metric": f"decode tok/s at batch {args.batch}, context {context} (Llama 3.2 1B layer sizes, random weights)",
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(sec * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids",
+        "dtype": args.dtype, "data": "synthetic: random weights N(0, 0.02), uniform random token ids"
+                + (", random cache contents" if synthetic else ""),
         "config": {
             "model": "llama-3.2-1b-sizes", "layers": args.layers, "layers_of_model": MODEL["num_hidden_layers"],
             "hidden_size": cfg.hidden_size, "heads": cfg.num_attention_heads, "kv_heads": cfg.num_key_value_heads,
             "head_dim": cfg.head_dim, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
             "tied_embeddings": cfg.tie_word_embeddings, "rope": "llama3 theta=500000 factor=32",
-            "global_batch": args.batch, "seq_len": CONTEXT, "kv_block": BLOCK_SIZE, "prefill_tokens": PREFILL_TOKENS,
+            "global_batch": args.batch, "seq_len": context, "kv_block": BLOCK_SIZE, "prefill_tokens": PREFILL_TOKENS,
             "parallelism": "single-gpu", "weight_bytes": wbytes, "kv_bytes_per_token": kvb,
             "weight_copies_in_streaming_order": runner.stream_copies,
         },
@@ -424,10 +522,12 @@ def main() -> int:
         line["prefill"] = {"value": round(PREFILL_TOKENS / psec, 1), "tokens": PREFILL_TOKENS, "ms": round(psec * 1e3, 3),
                            "frac": round(flops / psec / PEAK_FLOPS[args.dtype], 4)}
         points = {}
-        for b in (1, 64):
-            s, _ = time_decode(runner, b, args.steps, args.warmup, CONTEXT)
+        for b in more_batches:
+            s, _ = time_decode(runner, b, args.steps, args.warmup, context, synthetic_cache=synthetic)
             points[f"decode_b{b}"] = round(b / s, 1)
-        points["engine_b8"] = round(args.batch / time_engine_decode(runner, args.batch, args.steps, args.warmup, CONTEXT), 1)
+        if not synthetic:
+            points[f"engine_b{args.batch}"] = round(
+                args.batch / time_engine_decode(runner, args.batch, args.steps, args.warmup, context), 1)
         line["points"] = points
     print(json.dumps(line), flush=True)
     return 0

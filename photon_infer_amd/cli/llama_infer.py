@@ -12,15 +12,13 @@ from __future__ import annotations
 
 import argparse
 import sys
-import tempfile
 import time
 from typing import List, Optional
 
 from ..engine import ContinuousBatchEngine, EngineOptions
 from ..errors import PhotonError
-from ..registry import config_from_dict
 from ..tokenizer import TikTokenizer
-from ..weights import write_random_model
+from ..weights import random_model_folder
 
 DEFAULT_TURNS = ["My name is Lummy. Remember that.", "What is my name?"]   # demo/llama_infer.cpp:245,259
 
@@ -56,15 +54,9 @@ def build_parser() -> argparse.ArgumentParser:
 def _model_folder(args) -> str:
     if not args.random_weights:
         return args.model_dir
-    import json
-    import os
-    path = args.model_dir
-    cfg_path = os.path.join(path, "config.json") if os.path.isdir(path) else path
-    with open(cfg_path) as f:
-        cfg = config_from_dict(json.load(f), cfg_path)
-    out = tempfile.mkdtemp(prefix="photon_random_")
+    out = random_model_folder(args.model_dir, seed=args.seed, std=args.weight_std)
     print(f"Writing random weights (seed {args.seed}) to: {out}")
-    return write_random_model(cfg, out, seed=args.seed, std=args.weight_std)
+    return out
 
 
 def _prompts(args, tok: Optional[TikTokenizer]) -> List[tuple]:

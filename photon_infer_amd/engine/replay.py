@@ -16,6 +16,7 @@ from __future__ import annotations
 
 import json
 import os
+import shutil
 import sys
 from typing import IO, Optional
 
@@ -80,11 +81,26 @@ def main(argv=None) -> int:
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens live requests hold at any time, each rounded up to a multiple of 64")
     ap.add_argument("--block-size", type=int, default=16, help="tokens per cache page (divides 64)")
+    ap.add_argument("--random-weights", action="store_true",
+                    help="--model names a bare config.json (or a folder that holds only one); weights are drawn from --seed")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--weight-std", type=float, default=0.02)
     args = ap.parse_args(argv)
+    scratch = None
     try:
-        runner = make_runner(args.model, args.dtype, args.max_tokens, args.block_size)
+        model = args.model
+        if args.random_weights:
+            from ..weights import random_model_folder
+            model = scratch = random_model_folder(args.model, seed=args.seed, std=args.weight_std)
+        runner = make_runner(model, args.dtype, args.max_tokens, args.block_size)
+        if scratch is not None:       # the weights are on the device now
+            shutil.rmtree(scratch, ignore_errors=True)
+            scratch = None
         replay(runner, sys.stdin, args.out, sys.stdout)
     except PhotonError as e:
         print(f"trace_run: {e}", file=sys.stderr, flush=True)
         return 1
+    finally:
+        if scratch is not None:
+            shutil.rmtree(scratch, ignore_errors=True)
     return 0

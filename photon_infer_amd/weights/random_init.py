@@ -61,3 +61,16 @@ def write_random_model(config, out_dir: str, seed: int = 0, std: float = 0.02, n
     write_safetensors(os.path.join(out_dir, "model.safetensors"), tensors,
                       {"format": "pt", "seed": str(seed), "std": str(std), "norm_init": norm_init})
     return out_dir
+
+
+def random_model_folder(config_path: str, seed: int = 0, std: float = 0.02, norm_init: str = "ones") -> str:
+    """A fresh temporary model folder with random weights for the bare configuration at
+    ``config_path`` (a config.json file, or a folder that holds one).  The caller removes it."""
+    import tempfile
+
+    from ..registry import config_from_dict
+
+    path = os.path.join(config_path, "config.json") if os.path.isdir(config_path) else config_path
+    with open(path, encoding="utf-8") as f:
+        config = config_from_dict(json.load(f), path)
+    return write_random_model(config, tempfile.mkdtemp(prefix="photon_random_"), seed=seed, std=std, norm_init=norm_init)

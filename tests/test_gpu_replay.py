@@ -273,6 +273,27 @@ def test_the_command_itself(model_dirs, tmp_path, dtype):
     check(got, model_dirs["B"], reqs, dtype, "command")
 
 
+def test_the_command_from_a_bare_configuration_and_a_seed(tmp_path):
+    """--random-weights: the model is a config.json alone; the weights are those that the
+    random-weights mode writes for that configuration and seed."""
+    from photon_infer_amd.config import LlamaConfig
+    from photon_infer_amd.weights import write_random_model
+
+    (tmp_path / "bare").mkdir()
+    (tmp_path / "bare" / "config.json").write_text(json.dumps(ALL["B"][0]))
+    written = write_random_model(LlamaConfig.from_dict(ALL["B"][0]), str(tmp_path / "written"), seed=9, std=0.05)
+    reqs = requests_for("B", [41, 18], seed=8)
+    steps = mixed_trace(reqs, {"r0": [16, 3], "r1": [1, 7]})
+    for model in (str(tmp_path / "bare"), str(tmp_path / "bare" / "config.json")):
+        out = tmp_path / ("out_" + os.path.basename(model))
+        proc = subprocess.run(
+            [os.path.join(ROOT, "bin", "trace_run"), "--model", model, "--random-weights", "--seed", "9", "--weight-std", "0.05",
+             "--dtype", "float32", "--out", str(out), "--max-tokens", str(live_token_need(steps))],
+            input="\n".join(json.dumps(s) for s in steps) + "\n", capture_output=True, text=True, timeout=300)
+        assert proc.returncode == 0, proc.stderr[-2000:]
+        check(collect_logits(steps, str(out), ALL["B"][0]["vocab_size"]), written, reqs, "float32", "random weights")
+
+
 def test_the_command_reports_bad_models(tmp_path):
     (tmp_path / "config.json").write_text(json.dumps(dict(ALL["A"][0], architectures=["NopeForCausalLM"])))
     proc = subprocess.run(
