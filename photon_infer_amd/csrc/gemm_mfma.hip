@@ -20,6 +20,7 @@
 // accumulates over k in the same order whatever the other rows are.
 #include <type_traits>
 
+#include "addressing.h"
 #include "mfma.h"
 
 PI_DEFINE_MODULE(bf16)
@@ -127,11 +128,11 @@ __device__ inline void store_rows32(float* patch, const f32x16_t& acc0, const f3
 // Global loads go through buffer descriptors: a scalar base (the block's first row at its first
 // k), a byte length, and per-lane 32-bit offsets.  An offset at or beyond the length reads
 // zeros, which is how rows beyond the matrix and k beyond the range are filled, without a branch.
-#define PI_OUT_OF_RANGE 0x7ffffff0u
 #if defined(__HIP_DEVICE_COMPILE__)
-__device__ inline __amdgpu_buffer_rsrc_t operand_descriptor(const bf16_t* base, long bytes) {
+__device__ inline __amdgpu_buffer_rsrc_t operand_descriptor(const bf16_t* operand, addressing::Descriptor d) {
   // made scalar by hand so that the loads take the descriptor from scalar registers
-  const uint64_t v = reinterpret_cast<uint64_t>(base);
+  const long bytes = d.bytes;
+  const uint64_t v = reinterpret_cast<uint64_t>(operand + d.base);
   const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v));
   const uint32_t hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
   void* p = reinterpret_cast<void*>((static_cast<uint64_t>(hi) << 32) | lo);
@@ -176,31 +177,29 @@ __global__ __launch_bounds__(256) void gemm_mfma_kernel(void* __restrict__ Cv, l
   // range take an offset outside the descriptor and arrive as zeros.
   const int a_rows = (int)min((long)BM, M - m0), w_rows = (int)min((long)BN, N - n0);
 #if defined(__HIP_DEVICE_COMPILE__)
-  const __amdgpu_buffer_rsrc_t a_src = operand_descriptor(A + m0 * lda + k_lo, ((long)(a_rows - 1) * lda + (k_hi - k_lo)) * 2);
-  const __amdgpu_buffer_rsrc_t w_src = operand_descriptor(W + n0 * ldw + k_lo, ((long)(w_rows - 1) * ldw + (k_hi - k_lo)) * 2);
+  const __amdgpu_buffer_rsrc_t a_src = operand_descriptor(A, addressing::tile_descriptor(m0, lda, k_lo, k_hi, a_rows));
+  const __amdgpu_buffer_rsrc_t w_src = operand_descriptor(W, addressing::tile_descriptor(n0, ldw, k_lo, k_hi, w_rows));
 #endif
   unsigned a_off[4], w_off[4];
-  int piece_k[4];                           // first k (inside a slab) of the piece this lane fetches
+  int piece_k[4];                           // the piece (8 k) of a slab's row that this lane fetches
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     const int row = (wave * 4 + p) * 8 + lane / 8;
-    const int piece = (lane % 8) ^ ((row >> 1) & 7);
-    piece_k[p] = piece * 8;
-    a_off[p] = row < a_rows ? (unsigned)(row * (int)lda + piece * 8) * 2u : PI_OUT_OF_RANGE;
-    w_off[p] = row < w_rows ? (unsigned)(row * (int)ldw + piece * 8) * 2u : PI_OUT_OF_RANGE;
+    const int piece = addressing::tile_piece(lane, row);
+    piece_k[p] = piece;
+    a_off[p] = addressing::tile_lane_offset(row, a_rows, lda, piece);
+    w_off[p] = addressing::tile_lane_offset(row, w_rows, ldw, piece);
   }
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
   auto load_slab = [&](int k0, int buf) {
     // k0 is relative to k_lo; a lane's 8 k of the slab may lie beyond the range (last slab)
-    const unsigned kb = (unsigned)k0 * 2u;
 #if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
-      const bool k_in = k0 + piece_k[p] < k_hi - k_lo;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(a_src, (lds_ptr_t)(As + buf * TILE + (wave * 4 + p) * 8 * ROW), 16,
-                                               k_in ? a_off[p] + kb : PI_OUT_OF_RANGE, 0, 0, 0);
+                                               addressing::tile_slab_offset(a_off[p], k0, piece_k[p], k_hi - k_lo), 0, 0, 0);
       __builtin_amdgcn_raw_ptr_buffer_load_lds(w_src, (lds_ptr_t)(Ws + buf * TILE + (wave * 4 + p) * 8 * ROW), 16,
-                                               k_in ? w_off[p] + kb : PI_OUT_OF_RANGE, 0, 0, 0);
+                                               addressing::tile_slab_offset(w_off[p], k0, piece_k[p], k_hi - k_lo), 0, 0, 0);
     }
 #endif
   };
@@ -343,21 +342,21 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
   // so that the fragment reads of sixteen neighbouring rows fall on all 64 banks.
   const int a_rows = (int)min((long)GM, M - m0), w_rows = (int)min((long)GN, N - n0);
 #if defined(__HIP_DEVICE_COMPILE__)
-  const __amdgpu_buffer_rsrc_t a_src = operand_descriptor(A + m0 * lda + k_lo, ((long)(a_rows - 1) * lda + (k_hi - k_lo)) * 2);
-  const __amdgpu_buffer_rsrc_t w_src = operand_descriptor(W + n0 * ldw + k_lo, ((long)(w_rows - 1) * ldw + (k_hi - k_lo)) * 2);
+  const __amdgpu_buffer_rsrc_t a_src = operand_descriptor(A, addressing::tile_descriptor(m0, lda, k_lo, k_hi, a_rows));
+  const __amdgpu_buffer_rsrc_t w_src = operand_descriptor(W, addressing::tile_descriptor(n0, ldw, k_lo, k_hi, w_rows));
 #endif
   unsigned a_off[4], w_off[4];
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     const int row = (wave * 4 + p) * 8 + lane / 8;
-    const int piece = (lane % 8) ^ ((row >> 1) & 7);
-    a_off[p] = (unsigned)(min(row, a_rows - 1) * (int)lda + piece * 8) * 2u;
-    w_off[p] = (unsigned)(min(row, w_rows - 1) * (int)ldw + piece * 8) * 2u;
+    const int piece = addressing::tile_piece(lane, row);
+    a_off[p] = addressing::big_lane_offset(row, a_rows, lda, piece);
+    w_off[p] = addressing::big_lane_offset(row, w_rows, ldw, piece);
   }
   const int slabs = (k_hi - k_lo) / BK;
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
   auto load_slab = [&](int s, int buf) {
-    const int kbytes = min(s, slabs - 1) * BK * 2;     // past the last slab: read it again, unused
+    const int kbytes = addressing::big_slab_bytes(s, slabs);     // past the last slab: read it again, unused
 #if defined(__HIP_DEVICE_COMPILE__)
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
@@ -463,9 +462,9 @@ static int launch(void* C, long ldc, const void* A, long lda, const void* W, lon
     if (e != hipSuccess) return pi_fail("gemm_mfma: cannot reserve %zu bytes of LDS: %s", kLdsBytes, hipGetErrorString(e));
     configured = true;
   }
-  int kps = ceil_div(K, splits);
-  kps = ((kps + BK - 1) / BK) * BK;
-  splits = ceil_div(K, kps);
+  const addressing::KSplit cut = addressing::cut_k(K, splits, BK);
+  const int kps = cut.k_per_block;
+  splits = cut.splits;
   const long big_tiles = (long)ceil_div(M, GM) * ceil_div(N, GN);
   if (big_tiles * splits >= BIG_MIN_TILES && big_tiles < 2147483647L && K % BK == 0) {
     static bool big_configured = false;
@@ -488,9 +487,7 @@ static int launch(void* C, long ldc, const void* A, long lda, const void* W, lon
 // Pieces a k-split into `splits` makes (the kernel rounds a split's range up to whole slabs).
 extern "C" int pi_gemm_mfma_pieces(int K, int splits) {
   if (splits < 1 || K < 1) return 0;
-  int kps = ceil_div(K, splits);
-  kps = ((kps + BK - 1) / BK) * BK;
-  return ceil_div(K, kps);
+  return addressing::cut_k(K, splits, BK).splits;
 }
 
 // epilogue: 0 store bf16, 1 store f32, 2 add into f32, 3 SwiGLU (W rows interleaved by 16; C is [M, N / 2] bf16)

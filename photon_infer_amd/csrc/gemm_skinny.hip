@@ -16,13 +16,14 @@
 // same 16 features; no k-split over blocks in that case).
 #include <type_traits>
 
+#include "addressing.h"
 #include "mfma.h"
 
 enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACCUM = 2, EPI_SWIGLU = 3 };
 
 #define ROWS_PER_BLOCK 32
 #define RANGES_ROW_TILES 4      // row tiles per wave where the key ranges are merged on the way in (fewer blocks repeat the merge)
-#define KSTEP 64
+#define KSTEP addressing::KSTEP
 #define SHARED_FROM_TOKENS 32   // more tokens than this: the kernel that shares an activation tile per block
 #define SHARED_DEPTH 4          // k steps of loads a wave keeps in flight (measured: more is slower)
 
@@ -137,22 +138,16 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
   const int splits = gridDim.y;
 
   // this wave's k-range: a quarter (rounded up to whole steps) of the block's range
-  const int kb0 = blockIdx.y * k_per_block;
-  const int kb1 = min(K, kb0 + k_per_block);
-  const int per_wave = ((kb1 - kb0 + 4 * KSTEP - 1) / (4 * KSTEP)) * KSTEP;
-  const int k0 = kb0 + wave * per_wave;
-  const int k1 = min(kb1, k0 + per_wave);
+  const addressing::WaveRange range = addressing::skinny_wave_range(K, k_per_block, blockIdx.y, wave);
+  const int k0 = range.k0, k1 = range.k1;
 
   // rows beyond N read the last valid row; their results are never stored.  `tiled`: W is the
   // copy in the order this kernel reads (see pi_gemm_skinny): 16 rows x 64 k are 2 KB in a row,
   // one load instruction's 1 KB after the other, so a k step of 64 moves by 1,024 elements and
   // the step's second fragment lies 512 elements behind the first.
-  const int k_mul = tiled ? 16 : 1, h_mul = tiled ? 512 : 8;
   const bf16_t* wrow[RT];
 #pragma unroll
-  for (int t = 0; t < RT; ++t)
-    wrow[t] = tiled ? W + min(n0 / 16 + t, (long)N / 16 - 1) * (K / 64) * 1024 + lg * 128 + lr * 8
-                    : W + min(n0 + t * 16 + lr, (long)N - 1) * ldw + lg * 16;
+  for (int t = 0; t < RT; ++t) wrow[t] = W + addressing::skinny_w_base(tiled, n0, t, lr, lg, N, K, ldw);
 
   // Activations of a k step: load instruction i brings tokens 8i .. 8i+7, lane j the 16-byte
   // piece j % 8 of token 8i + j / 8.  Tokens beyond M are not loaded: what LDS holds for them
@@ -164,7 +159,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
 #pragma unroll
   for (int i = 0; i < MB * 2; ++i) {
     const int token = i * 8 + xt;
-    xsrc[i] = X + (long)min(token, M - 1) * ldx + xp * 8;
+    xsrc[i] = X + addressing::skinny_x_base(token, M, ldx, xp);
     xdst[i] = ((token / 16) * 8 + xp) * 16 + ((token + 2 * xp) & 15);
   }
   u32x4_t* xs = lds.xs[wave];
@@ -189,12 +184,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
     for (int t = 0; t < RT; ++t)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        // a piece beyond k1 is fetched from the range's first 8 elements instead (k0 + 8 <= k1:
-        // both are multiples of 8), which lie inside the row whatever the lane's own offset
-        // (a tiled matrix has whole steps only)
-        if (whole) w[t][h] = load_frag(wrow[t] + (long)kk * k_mul + h * h_mul);
-        else w[t][h] = load_frag(wrow[t] + (kk + lg * 16 + h * 8 < k1 ? kk + h * 8 : k0 - lg * 16));
-        if (!whole && kk + lg * 16 + h * 8 >= k1) w[t][h] = zero_frag();
+        // a piece beyond k1 is fetched from a stand-in address inside the row and counts as zero
+        w[t][h] = load_frag(wrow[t] + addressing::skinny_w_step(tiled, whole, kk, h, lg, k0, k1));
+        if (!addressing::skinny_w_used(whole, kk, h, lg, k1)) w[t][h] = zero_frag();
       }
     if constexpr (RANGES) {
       // The 64 features of this step belong to one head (head_dim is a multiple of 64).  Lane
@@ -216,7 +208,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(void* __restrict__ Cv,
 #pragma unroll
       for (int i = 0; i < MB * 2; ++i)
         if (i == 0 || i < x_loads) {
-          xg[i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + (x_ok ? kk : k0 - xp * 8));
+          xg[i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + addressing::skinny_x_step(whole, kk, xp, k0, k1));
           if (!x_ok) xg[i] = u32x4_t{0u, 0u, 0u, 0u};
         }
 #pragma unroll
@@ -313,12 +305,11 @@ __global__ __launch_bounds__(256) void gemm_skinny_shared_kernel(void* __restric
   const int splits = gridDim.y;
   const int kb0 = blockIdx.y * k_per_block;
   const int kb1 = min(K, kb0 + k_per_block);
-  const int steps = (kb1 - kb0 + KSTEP - 1) / KSTEP;
-  auto k_of = [&](const int s) { return kb0 + min(s, steps - 1) * KSTEP; };   // steps beyond the last are fetched, never used
+  const int steps = addressing::shared_steps(kb0, kb1);
+  auto k_of = [&](const int s) { return addressing::shared_k_of(kb0, steps, s); };   // steps beyond the last are fetched, never used
 
   // rows beyond N and tokens beyond M read the last valid one; their results are never stored
-  const bf16_t* wrow = tiled ? W + min(n0 / 16 + wave, (long)N / 16 - 1) * (K / 64) * 1024 + lg * 128 + lr * 8     // see gemm_skinny_kernel
-                             : W + min(n0 + wave * 16 + lr, (long)N - 1) * ldw;
+  const bf16_t* wrow = W + addressing::shared_w_base(tiled, n0, wave, lr, lg, N, K, ldw);     // see gemm_skinny_kernel
   const int xp = tid % 8;
   const bf16_t* xsrc[XL];
   int xdst[XL];
@@ -326,7 +317,7 @@ __global__ __launch_bounds__(256) void gemm_skinny_shared_kernel(void* __restric
 #pragma unroll
   for (int i = 0; i < XL; ++i) {
     const int token = i * 32 + tid / 8;
-    xsrc[i] = X + (long)min(token, M - 1) * ldx;
+    xsrc[i] = X + addressing::shared_x_base(token, M, ldx);
     xdst[i] = ((token / 16) * 8 + xp) * 16 + ((token + 2 * xp) & 15);
     xmine[i] = token < MB * 16;
   }
@@ -347,9 +338,9 @@ __global__ __launch_bounds__(256) void gemm_skinny_shared_kernel(void* __restric
   auto fetch = [&](const int s, const int j) {
     const int kk = k_of(s);
 #pragma unroll
-    for (int i = 0; i < XL; ++i) xq[j][i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + min(kk + xp * 8, kb1 - 8));
+    for (int i = 0; i < XL; ++i) xq[j][i] = *reinterpret_cast<const u32x4_t*>(xsrc[i] + addressing::shared_x_step(kk, xp, kb1));
 #pragma unroll
-    for (int h = 0; h < 2; ++h) wq[j][h] = load_frag(wrow + (tiled ? (long)kk * 16 + h * 512 : (long)min(kk + lg * 16 + h * 8, kb1 - 8)));
+    for (int h = 0; h < 2; ++h) wq[j][h] = load_frag(wrow + addressing::shared_w_step(tiled, kk, h, lg, kb1));
   };
 #pragma unroll
   for (int j = 0; j < DEPTH; ++j) fetch(j, j);
@@ -496,9 +487,9 @@ extern "C" int pi_gemm_skinny(void* C, int epilogue, long ldc, const void* X, lo
   PI_REQUIRE(splits >= 1 && splits <= 65535, "gemm_skinny: bad split count %d", splits);
   PI_REQUIRE(epilogue != EPI_SWIGLU || (splits == 1 && N % 32 == 0), "gemm_skinny: the SwiGLU epilogue needs one split and N (%d) a multiple of 32", N);
   const int groups = ceil_div(N, pi_gemm_skinny_rows_per_block(M));
-  int kpb = ceil_div(K, splits);
-  kpb = ((kpb + KSTEP - 1) / KSTEP) * KSTEP;
-  splits = ceil_div(K, kpb);                      // no empty splits
+  const addressing::KSplit cut = addressing::cut_k(K, splits, KSTEP);
+  const int kpb = cut.k_per_block;
+  splits = cut.splits;                            // no empty splits
   if (splits > 1)
     PI_REQUIRE(part && part_elems >= (long)splits * M * N, "gemm_skinny: workspace too small (%ld floats for %ld)", part_elems, (long)splits * M * N);
   if (splits_out) *splits_out = splits;
@@ -536,9 +527,9 @@ extern "C" int pi_gemm_skinny_ranges(void* C, int epilogue, long ldc, const void
   const long K = (long)heads * head_dim;
   PI_REQUIRE(K < (1L << 30), "gemm_skinny_ranges: k too long");
   PI_REQUIRE(!tiled || N % 16 == 0, "gemm_skinny_ranges: a tiled weight matrix needs N (%d) a multiple of 16", N);
-  int kpb = ceil_div((int)K, splits);
-  kpb = ((kpb + 4 * KSTEP - 1) / (4 * KSTEP)) * (4 * KSTEP);     // a block's four waves take whole steps
-  splits = ceil_div((int)K, kpb);
+  const addressing::KSplit cut = addressing::cut_k((int)K, splits, 4 * KSTEP);     // a block's four waves take whole steps
+  const int kpb = cut.k_per_block;
+  splits = cut.splits;
   if (splits > 1)
     PI_REQUIRE(part && part_elems >= (long)splits * M * N, "gemm_skinny_ranges: workspace too small (%ld floats for %ld)", part_elems, (long)splits * M * N);
   if (splits_out) *splits_out = splits;
