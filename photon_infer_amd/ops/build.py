@@ -33,7 +33,7 @@ MODULES: Dict[str, List[str]] = {
     # host only: the engine for C / C++ programs (hosts an interpreter; links libpython)
     "api": ["api/photon_engine.cpp"],
 }
-HEADERS = ["common.h", "mfma.h", "attention_mfma.h", "sampling.h"]
+HEADERS = ["common.h", "mfma.h", "addressing.h", "attention_mfma.h", "sampling.h"]
 HOST_MODULES = {"runtime", "api"}
 HOST_HEADERS = {"api": ["api/photon_engine.h"]}
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-Wall"]
