@@ -15,14 +15,14 @@ import torch
 
 class StateSlots:
     def __init__(self, specs: Sequence[Tuple[int, object]], max_slots: int, device):
-        """``specs``: (run-order index, StateSpec) pairs."""
+        """``specs``: (key, StateSpec) pairs; a key names the mixer that owns the state (run-order entry, mixer index)."""
         self.max_slots = int(max_slots)
-        self.slabs: Dict[int, torch.Tensor] = {
+        self.slabs: Dict[object, torch.Tensor] = {
             entry: torch.zeros((self.max_slots, *spec.shape), dtype=spec.dtype, device=device)
             for entry, spec in specs
         }
 
-    def get(self, entry: int):
+    def get(self, entry):
         return self.slabs.get(entry)
 
     def clear(self, slot: int) -> None:

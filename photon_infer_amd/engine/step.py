@@ -120,9 +120,10 @@ class ModelRunner:
         # what the mixers want planned on the host per step (equal planners are kept once)
         self.planners = []
         for e in self.spec.run_order:
-            planner = self.spec.layers[e.layer][1].mixer.step_planner(self.page_size)
-            if planner is not None and planner not in self.planners:
-                self.planners.append(planner)
+            for mixer in self.spec.layers[e.layer][1].mixers():
+                planner = mixer.step_planner(self.page_size)
+                if planner is not None and planner not in self.planners:
+                    self.planners.append(planner)
         # a decode step is captured as a HIP graph only when every part promises that its launches
         # do not depend on host-side values of the step
         self.graph_safe = self.model.graph_safe
@@ -167,9 +168,8 @@ class ModelRunner:
         self.page_size = int(o.block_size)
         if self.page_size <= 0 or o.max_batch <= 0:
             raise RequestError("block_size and max_batch must be positive")
-        # bytes of keys and values that one page holds over all layers that own pages
-        itemsize = torch.empty((), dtype=self.dtype).element_size()
-        page_bytes = sum(2 * nkv * hd * self.page_size * itemsize for g in self.plan.groups for nkv, hd in g.kv_shapes)
+        # bytes that one page holds over all mixers that own pages (whatever each keeps per token)
+        page_bytes = sum(t.page_bytes(self.page_size, self.dtype) for g in self.plan.groups for owner in g.tensors for t in owner)
         free = self._free_device_bytes()
         if o.num_blocks is not None or o.max_cache_tokens is not None:
             num_pages = int(o.num_blocks) if o.num_blocks is not None else max(1, -(-int(o.max_cache_tokens) // self.page_size))
@@ -198,26 +198,33 @@ class ModelRunner:
         self.cache = CacheManager([g.window for g in self.plan.groups], self.page_size, num_pages,
                                   o.max_batch, self.max_model_len)
         self.states = StateSlots(self.plan.states, o.max_batch, self.device)
-        # one K and one V pool per run-order entry that owns pages: keys [pages, kv_heads, page,
-        # head_dim], values [pages, kv_heads, head_dim, page] (the layout the kernels contract in)
-        pools: Dict[int, tuple] = {}
+        # one pool per paged tensor of every mixer that owns pages, [pages, *page shape]: for
+        # attention, keys [pages, kv_heads, page, head_dim] and values [pages, kv_heads, head_dim,
+        # page] (the layout the kernels contract in)
+        pools: Dict[tuple, Dict[str, torch.Tensor]] = {}
         try:
             for g in self.plan.groups:
-                for entry, (nkv, hd) in zip(g.entries, g.kv_shapes):
-                    pools[entry] = (torch.zeros((num_pages, nkv, self.page_size, hd), dtype=self.dtype, device=self.device),
-                                    torch.zeros((num_pages, nkv, hd, self.page_size), dtype=self.dtype, device=self.device))
+                for owner, tensors in zip(g.owners, g.tensors):
+                    pools[owner] = {t.name: torch.zeros((num_pages, *t.page_shape(self.page_size)), dtype=t.dtype or self.dtype,
+                                                        device=self.device) for t in tensors}
         except torch.OutOfMemoryError as e:
             pools.clear()
             raise OutOfMemoryError(f"the cache pools ({num_pages} pages of {page_bytes} bytes) do not fit the device: {e}") from None
-        self.layer_caches: List[LayerCache] = []
+        # what each run-order entry's block is handed: its mixer's view, or a list of views when
+        # the block has several mixers
+        self.layer_caches: List = []
         for i, e in enumerate(self.spec.run_order):
-            owner = i if e.cache_of is None else e.cache_of
-            lc = LayerCache(writes=e.cache_of is None, state=self.states.get(owner))
-            if owner in pools:
-                lc.group = self.plan.group_of_entry[owner]
-                lc.k, lc.v = pools[owner]
-                lc.page_size = self.page_size
-            self.layer_caches.append(lc)
+            views = []
+            for j, _mixer in enumerate(self.spec.layers[e.layer][1].mixers()):
+                owner = self.plan.owner_of[(i, j)]
+                lc = LayerCache(writes=e.cache_of is None, state=self.states.get(owner))
+                if owner in pools:
+                    lc.group = self.plan.group_of[owner]
+                    lc.tensors = pools[owner]
+                    lc.k, lc.v = lc.tensors.get("k"), lc.tensors.get("v")
+                    lc.page_size = self.page_size
+                views.append(lc)
+            self.layer_caches.append(views[0] if len(views) == 1 else (views or LayerCache()))
 
     # ------------------------------------------------------------------ request life cycle
     def admit(self, rid: Hashable) -> int:

@@ -1,6 +1,7 @@
 """Parts that layers are put together from; importing the package registers the built-in ones."""
 from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Block, FeedForward,
-                   KVCacheSpec, LayerCache, Mixer, Norm, Part, PositionEncoding, StateSpec, StepContext)
+                   KVCacheSpec, LayerCache, Mixer, Norm, PAGE, PagedCacheSpec, PagedTensor, Part, PositionEncoding, StateSpec,
+                   StepContext)
 from .norm import RMSNorm
 from .rope import RotaryEmbedding, rope_frequencies
 from .attention import PagedAttention
@@ -11,7 +12,7 @@ from .model import CachePlan, DecoderModel, ModelSpec, RunEntry, plan_cache
 
 __all__ = [
     "BLOCKS", "FEED_FORWARDS", "MIXERS", "NORMS", "POSITION_ENCODINGS", "Block", "FeedForward",
-    "KVCacheSpec", "LayerCache", "Mixer", "Norm", "Part", "PositionEncoding", "StateSpec",
+    "KVCacheSpec", "LayerCache", "Mixer", "Norm", "PAGE", "PagedCacheSpec", "PagedTensor", "Part", "PositionEncoding", "StateSpec",
     "StepContext", "RMSNorm", "RotaryEmbedding", "rope_frequencies", "PagedAttention", "SwiGLU",
     "PreNormBlock", "LMHead", "TokenEmbedding", "CachePlan", "DecoderModel", "ModelSpec",
     "RunEntry", "plan_cache",

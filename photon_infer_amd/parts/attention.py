@@ -111,7 +111,7 @@ class PagedAttention(Mixer):
                                                         leave_ranges=self.w_o.numel() * self.w_o.element_size())
             if done:
                 # the output, or its key ranges still to be merged, which the product does as it reads them
-                ops.gemm(x, done if isinstance(done, ops.KeyRanges) else attn, self.w_o, accumulate=True, may_defer=True, ws=ws)
+                ops.gemm(x, done if isinstance(done, ops.KeyRanges) else attn, self.w_o, accumulate=True, may_defer=getattr(ctx, "may_defer", False), ws=ws)
                 return
         if qkv is not None and not isinstance(qkv, torch.Tensor):
             # the projection is still in pieces (split over k): the rotation kernel sums them
@@ -138,8 +138,8 @@ class PagedAttention(Mixer):
             self.num_heads, self.num_kv_heads, self.head_dim, cache.page_size,
             self.scale, self.window or 0, ws,
         )
-        # the block's next norm reads x, so the product may stay in pieces until then
-        ops.gemm(x, attn, self.w_o, accumulate=True, may_defer=True, ws=ws)
+        # where the arrangement allows it, the product stays in pieces for the stream's next reader
+        ops.gemm(x, attn, self.w_o, accumulate=True, may_defer=getattr(ctx, "may_defer", False), ws=ws)
 
 
 MIXERS.register("attention", PagedAttention)

@@ -16,7 +16,7 @@ a mixer or feed-forward reads ``h`` and *adds* its result into ``x``.
 from __future__ import annotations
 
 from dataclasses import dataclass, field
-from typing import Any, Callable, Dict, List, Optional, Sequence
+from typing import Any, Callable, Dict, List, Optional, Sequence, Tuple
 
 import torch
 
@@ -25,17 +25,56 @@ from ..weights.loader import TensorSpec
 
 
 # --------------------------------------------------------------------------- cache needs
+PAGE = -1     # in a paged tensor's shape: the axis that holds a page's tokens
+
+
+@dataclass(frozen=True)
+class PagedTensor:
+    """One tensor that a mixer keeps per token, in pages: the shape of one page of it, with ``PAGE``
+    standing for the page's tokens, e.g. keys ``(kv_heads, PAGE, head_dim)``, values transposed
+    ``(kv_heads, head_dim, PAGE)``, one latent vector per token ``(PAGE, width)``.  The pool is
+    ``[pages, *shape]``.  ``dtype`` None: the compute dtype."""
+
+    name: str
+    shape: tuple
+    dtype: Optional[torch.dtype] = None
+
+    def page_shape(self, page_size: int) -> tuple:
+        if sum(1 for d in self.shape if d == PAGE) != 1:
+            raise UnsupportedModelError(f"paged tensor '{self.name}': its shape {self.shape} must name the page axis once")
+        return tuple(page_size if d == PAGE else int(d) for d in self.shape)
+
+    def page_bytes(self, page_size: int, compute_dtype: torch.dtype) -> int:
+        n = 1
+        for d in self.page_shape(page_size):
+            n *= d
+        return n * torch.empty((), dtype=self.dtype or compute_dtype).element_size()
+
+
+@dataclass(frozen=True)
+class PagedCacheSpec:
+    """What a mixer keeps per token, in pages: any number of named tensors, each with its own
+    shape and layout.  ``window`` = None keeps every token; an integer W keeps the last W
+    positions, so the cache manager may hand back pages that the window has passed.  Mixers with
+    the same window share a cache group (one page pool's bookkeeping, one block table)."""
+
+    tensors: Tuple[PagedTensor, ...]
+    window: Optional[int] = None
+
+
 @dataclass(frozen=True)
 class KVCacheSpec:
-    """Keys and values kept per token, in pages.
-
-    ``window`` = None keeps all keys; an integer W keeps the last W positions, so the
-    cache manager may hand back pages that the window has passed.
-    """
+    """The usual case of ``PagedCacheSpec``: keys ``k`` [kv_heads, page, head_dim] and values
+    ``v`` transposed [kv_heads, head_dim, page] (the layout the attention kernels contract in)."""
 
     num_kv_heads: int
     head_dim: int
     window: Optional[int] = None
+
+    @property
+    def tensors(self) -> Tuple[PagedTensor, ...]:
+        return (PagedTensor("k", (self.num_kv_heads, PAGE, self.head_dim)),
+                PagedTensor("v", (self.num_kv_heads, self.head_dim, PAGE)))
 
 
 @dataclass(frozen=True)
@@ -74,6 +113,11 @@ class StepContext:
     max_kv_len: int = 0
     all_decode: bool = False
     host_slots: Sequence[int] = ()        # the requests' state slots, on the host
+    # Set by whoever arranges the parts, for the part that runs next: it may leave its update of
+    # the stream in pieces (``ops.gemm(..., may_defer=True)``) because the stream's next reader
+    # adds them.  False unless an arrangement says so, so a part never defers by itself.
+    may_defer: bool = False
+    after_block_consumes: bool = False    # set by the model per block: whoever reads the stream after this block adds pending pieces
     workspace: Any = None                 # the runner's ops.KernelWorkspace: scratch memory of the kernels
     plans: Dict[Any, Any] = field(default_factory=dict)     # step planner -> what it made for this step
     scratch: Dict[Any, Any] = field(default_factory=dict)   # what parts share within one step; emptied per step
@@ -84,11 +128,12 @@ class LayerCache:
     """The view of the cache manager that one entry of the run order gets."""
 
     group: int = -1                       # cache group of the pages (-1: no pages)
-    k: Optional[torch.Tensor] = None      # [pages, kv_heads, page_size, head_dim]
-    v: Optional[torch.Tensor] = None      # [pages, kv_heads, head_dim, page_size]
+    k: Optional[torch.Tensor] = None      # [pages, kv_heads, page_size, head_dim]   (= tensors["k"])
+    v: Optional[torch.Tensor] = None      # [pages, kv_heads, head_dim, page_size]   (= tensors["v"])
     page_size: int = 0
     writes: bool = True                   # False: reads another entry's cache
     state: Optional[torch.Tensor] = None  # [max_slots, *StateSpec.shape]
+    tensors: Dict[str, torch.Tensor] = field(default_factory=dict)   # every paged tensor by name: [pages, *page shape]
 
 
 # --------------------------------------------------------------------------- part bases
@@ -145,7 +190,8 @@ class PositionEncoding(Part):
 
 class Mixer(Part):
     def cache_spec(self):
-        """KVCacheSpec, StateSpec or None."""
+        """What the mixer keeps per request: ``KVCacheSpec`` / ``PagedCacheSpec`` (per token, in
+        pages), ``StateSpec`` (fixed size), or None."""
         return None
 
     def step_planner(self, page_size: int):
@@ -169,11 +215,23 @@ class FeedForward(Part):
 
 
 class Block(Part):
-    """An arrangement of norm(s), mixer and feed-forward around the residual stream."""
+    """An arrangement of norm(s), mixer(s) and feed-forward around the residual stream.
+
+    The stream a block receives is finished (no update pending) unless the block says that its
+    first reader adds pending pieces (``reads_deferred``), and no part inside it leaves an update
+    pending unless the block sets ``ctx.may_defer`` before calling it.  An arrangement that knows
+    nothing of deferred updates therefore never meets one."""
 
     mixer: Mixer
+    reads_deferred = False     # True: the block's first reader of the stream is a norm that adds pending pieces
 
-    def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
+    def mixers(self) -> List[Mixer]:
+        """The block's mixers, each with a cache or state of its own.  With more than one,
+        ``forward`` receives a list of ``LayerCache`` in this order instead of a single one."""
+        m = getattr(self, "mixer", None)
+        return [m] if m is not None else []
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, cache) -> None:
         raise NotImplementedError
 
 

@@ -38,16 +38,19 @@ class PreNormBlock(Block):
     def streamed_weights(self) -> List[torch.Tensor]:
         return [w for _, part in self._named for w in part.streamed_weights()]
 
+    @property
+    def reads_deferred(self) -> bool:
+        return bool(getattr(self.norm1, "consumes_deferred", False))
+
     def forward(self, x: torch.Tensor, ctx: StepContext, cache: LayerCache) -> None:
-        # A mixer or feed-forward may leave its update of x in pieces for the next norm to add
-        # (ops.gemm(..., may_defer=True)).  A norm that does not go through ops.rmsnorm gets
-        # the finished stream; mixers and feed-forwards always do, since a norm runs before them.
-        if not getattr(self.norm1, "consumes_deferred", False):
-            ops.materialize(x, ctx.workspace)
+        # A mixer or feed-forward may leave its update of x in pieces (ops.gemm(..., may_defer=True))
+        # when the stream's next reader adds them: norm2 after the mixer; after the feed-forward,
+        # whoever the model says reads the stream next.
+        ctx.may_defer = bool(getattr(self.norm2, "consumes_deferred", False))
         self.mixer.forward(self.norm1.forward(x, ctx), x, ctx, cache)
-        if not getattr(self.norm2, "consumes_deferred", False):
-            ops.materialize(x, ctx.workspace)
+        ctx.may_defer = ctx.after_block_consumes
         self.ffn.forward(self.norm2.forward(x, ctx), x, ctx)
+        ctx.may_defer = False
 
 
 BLOCKS.register("prenorm", PreNormBlock)

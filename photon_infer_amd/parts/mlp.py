@@ -61,7 +61,7 @@ class SwiGLU(FeedForward):
         act = torch.empty((h.shape[0], self.intermediate_size), dtype=self.dtype, device=h.device)
         ws = ctx.workspace if ctx is not None else None
         ops.gemm_swiglu(act, h, self.w_gate_up, self.interleave, ws=ws)
-        ops.gemm(x, act, self.w_down, accumulate=True, may_defer=True, ws=ws)   # the next norm reads x
+        ops.gemm(x, act, self.w_down, accumulate=True, may_defer=getattr(ctx, "may_defer", False), ws=ws)
 
 
 FEED_FORWARDS.register("swiglu", SwiGLU)

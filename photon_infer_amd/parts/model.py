@@ -16,7 +16,7 @@ import torch
 from .. import ops
 from ..errors import ConfigError
 from ..weights.loader import TensorSpec
-from .base import Block, KVCacheSpec, LayerCache, Norm, StateSpec, StepContext
+from .base import Block, KVCacheSpec, LayerCache, Norm, PagedCacheSpec, PagedTensor, StateSpec, StepContext
 from .embedding import LMHead, TokenEmbedding
 
 
@@ -62,50 +62,58 @@ class ModelSpec:
 
 
 # ------------------------------------------------------------------ what the cache must hold
+# A cache or a state belongs to one mixer of one run-order entry: the key (entry index, index of
+# the mixer among the block's ``mixers()``).
+CacheKey = Tuple[int, int]
+
+
 @dataclass(frozen=True)
 class CacheGroupPlan:
-    """Run-order entries whose keys/values live in pages of one pool."""
+    """Mixers whose paged tensors follow one block table (the same window)."""
 
     window: Optional[int]
-    entries: Tuple[int, ...]             # run-order indices that own K/V pages
-    kv_shapes: Tuple[Tuple[int, int], ...]  # (kv_heads, head_dim) per entry
+    owners: Tuple[CacheKey, ...]                        # the mixers that own pages
+    tensors: Tuple[Tuple[PagedTensor, ...], ...]        # per owner: what it keeps per token
 
 
 @dataclass(frozen=True)
 class CachePlan:
     groups: Tuple[CacheGroupPlan, ...]
-    states: Tuple[Tuple[int, StateSpec], ...]   # (run-order index, spec)
-    group_of_entry: Dict[int, int]
+    states: Tuple[Tuple[CacheKey, StateSpec], ...]
+    group_of: Dict[CacheKey, int]                       # also for mixers that read another entry's pages
+    owner_of: Dict[CacheKey, CacheKey]                  # whose cache or state a mixer uses (itself, or its ``cache_of`` entry's)
 
 
 def plan_cache(spec: ModelSpec) -> CachePlan:
-    """Group the run order's cache needs: one page pool per distinct window."""
-    by_window: Dict[Optional[int], List[Tuple[int, KVCacheSpec]]] = {}
-    states: List[Tuple[int, StateSpec]] = []
+    """Group the run order's cache needs: one block table per distinct window."""
+    by_window: Dict[Optional[int], List[Tuple[CacheKey, tuple]]] = {}
+    states: List[Tuple[CacheKey, StateSpec]] = []
+    owner_of: Dict[CacheKey, CacheKey] = {}
     for i, e in enumerate(spec.run_order):
-        mixer = spec.layers[e.layer][1].mixer
-        if e.cache_of is not None:
-            continue
-        if not getattr(mixer, "own_kv", True):
-            raise ConfigError(f"run order entry {i}: layer {e.layer} writes no keys or values of its own and "
-                              f"must name the entry whose cache it reads")
-        need = mixer.cache_spec()
-        if isinstance(need, KVCacheSpec):
-            by_window.setdefault(need.window, []).append((i, need))
-        elif isinstance(need, StateSpec):
-            states.append((i, need))
-        elif need is not None:
-            raise ConfigError(f"mixer of layer {e.layer} returned an unknown cache spec {need!r}")
-    groups, group_of_entry = [], {}
+        for j, mixer in enumerate(spec.layers[e.layer][1].mixers()):
+            if e.cache_of is not None:
+                owner_of[(i, j)] = (e.cache_of, j)
+                continue
+            owner_of[(i, j)] = (i, j)
+            if not getattr(mixer, "own_kv", True):
+                raise ConfigError(f"run order entry {i}: layer {e.layer} writes no keys or values of its own and "
+                                  f"must name the entry whose cache it reads")
+            need = mixer.cache_spec()
+            if isinstance(need, (KVCacheSpec, PagedCacheSpec)):
+                by_window.setdefault(need.window, []).append(((i, j), tuple(need.tensors)))
+            elif isinstance(need, StateSpec):
+                states.append(((i, j), need))
+            elif need is not None:
+                raise ConfigError(f"mixer {j} of layer {e.layer} returned an unknown cache spec {need!r}")
+    groups, group_of = [], {}
     for g, (window, items) in enumerate(sorted(by_window.items(), key=lambda kv: (kv[0] is not None, kv[0] or 0))):
-        groups.append(CacheGroupPlan(window, tuple(i for i, _ in items),
-                                     tuple((n.num_kv_heads, n.head_dim) for _, n in items)))
-        for i, _ in items:
-            group_of_entry[i] = g
-    for i, e in enumerate(spec.run_order):
-        if e.cache_of is not None and e.cache_of in group_of_entry:
-            group_of_entry[i] = group_of_entry[e.cache_of]
-    return CachePlan(tuple(groups), tuple(states), group_of_entry)
+        groups.append(CacheGroupPlan(window, tuple(k for k, _ in items), tuple(t for _, t in items)))
+        for k, _ in items:
+            group_of[k] = g
+    for key, owner in owner_of.items():
+        if owner in group_of:
+            group_of[key] = group_of[owner]
+    return CachePlan(tuple(groups), tuple(states), group_of, owner_of)
 
 
 # ------------------------------------------------------------------ the runnable model
@@ -130,18 +138,33 @@ class DecoderModel:
         for prefix, block in self.spec.layers:
             block.load(sub(prefix), dtype, device)
         self.final_norm.load(sub(self.spec.final_norm[0]), dtype, device)
-        self.head.load(sub(self.spec.head[0]), dtype, device, tied_weight=self.embedding.weight)
+        # a head that is tied takes the embedding's matrix itself
+        self.head.load(sub(self.spec.head[0]), dtype, device, tied_weight=getattr(self.embedding, "weight", None))
 
-    def forward(self, ctx: StepContext, caches: Sequence[LayerCache]) -> Optional[torch.Tensor]:
+    def forward(self, ctx: StepContext, caches: Sequence) -> Optional[torch.Tensor]:
         """Run the step's tokens through the run order; float32 logits [M, vocab] at
-        ``ctx.logit_rows`` (None when no row is wanted)."""
+        ``ctx.logit_rows`` (None when no row is wanted).  ``caches``: per run-order entry its
+        ``LayerCache`` (a list of them for a block of several mixers)."""
         ws = ctx.workspace
         ops.reset_deferred(ws)             # nothing of an earlier (failed) step may linger
         ctx.scratch.clear()
         x = self.embedding.forward(ctx.token_ids)
-        for i, entry in enumerate(self.spec.run_order):
-            self.blocks[entry.layer].forward(x, ctx, caches[i])
-        if ctx.logit_rows.shape[0] == 0:
+        order = self.spec.run_order
+        wanted = ctx.logit_rows.shape[0] > 0
+        for i, entry in enumerate(order):
+            block = self.blocks[entry.layer]
+            # A block meets an update of the stream that is still in pieces only if it says that
+            # its first reader adds them, and may leave one behind only for such a reader.
+            if not block.reads_deferred:
+                ops.materialize(x, ws)
+            if i + 1 < len(order):
+                ctx.after_block_consumes = bool(self.blocks[order[i + 1].layer].reads_deferred)
+            else:                          # the final norm; or nobody (the pieces are then dropped unread)
+                ctx.after_block_consumes = not wanted or bool(getattr(self.final_norm, "consumes_deferred", False))
+            ctx.may_defer = False
+            block.forward(x, ctx, caches[i])
+        ctx.may_defer = ctx.after_block_consumes = False
+        if not wanted:
             ops.discard_deferred(x, ws)    # the stream is not read again
             return None
         if not getattr(self.final_norm, "consumes_deferred", False):

@@ -239,8 +239,8 @@ def test_toy_mixer_with_state_registers_builds_and_steps(tmp_path):
     raw, W = P.read_model_folder(d)
     runner = ModelRunner(d, EngineOptions(dtype="float32", block_size=4, num_blocks=24, max_batch=2))
     # the plan: one page group (layer 1's; the last entry shares it), two state slabs (layer 0 runs twice)
-    assert len(runner.plan.groups) == 1 and runner.plan.groups[0].entries == (1,)
-    assert sorted(e for e, _ in runner.plan.states) == [0, 2]
+    assert len(runner.plan.groups) == 1 and runner.plan.groups[0].owners == ((1, 0),)
+    assert sorted(e for e, _ in runner.plan.states) == [(0, 0), (2, 0)]
     assert runner.layer_caches[3].k is runner.layer_caches[1].k and not runner.layer_caches[3].writes
     assert runner.layer_caches[0].state is not runner.layer_caches[2].state
     assert runner.states.bytes_per_slot == 2 * 49 * 4

@@ -141,7 +141,7 @@ def test_the_windows_matter_and_the_groups_are_three(toy):
     assert (wrong_edge[100:] - ref[100:]).abs().max() > fp32_tol(ref) * 3   # and one key too many, in float32
     runner = runner_for(d, "float32", 64)
     assert [g.window for g in runner.plan.groups] == [None, 24, 40]
-    assert [g.entries for g in runner.plan.groups] == [(0,), (2,), (1,)]
+    assert [g.owners for g in runner.plan.groups] == [((0, 0),), ((2, 0),), ((1, 0),)]
     assert len({id(lc.k) for lc in runner.layer_caches}) == 3
 
 
