@@ -448,7 +448,17 @@ __global__ __launch_bounds__(512) void gemm_mfma_big_kernel(void* __restrict__ C
 }
 
 static const size_t kBigLdsBytes = 4 * BIG_TILE_ELEMS * sizeof(uint16_t);   // 131,072 bytes
-#define BIG_MIN_TILES 192      // enough 256 x 256 tiles (times k pieces) to occupy most of the chip
+// enough 256 x 256 tiles (times k pieces) to occupy most of the chip: three quarters of its compute units
+static int big_min_tiles() {
+  static int units = 0;
+  if (units == 0) {
+    int device = 0, count = 0;
+    if (hipGetDevice(&device) != hipSuccess || hipDeviceGetAttribute(&count, hipDeviceAttributeMultiprocessorCount, device) != hipSuccess || count <= 0)
+      count = 256;
+    units = count;
+  }
+  return units * 3 / 4;
+}
 
 static const size_t kLdsBytes = 4 * TILE_ELEMS * sizeof(uint16_t);   // 65,536 bytes
 
@@ -466,7 +476,7 @@ static int launch(void* C, long ldc, const void* A, long lda, const void* W, lon
   const int kps = cut.k_per_block;
   splits = cut.splits;
   const long big_tiles = (long)ceil_div(M, GM) * ceil_div(N, GN);
-  if (big_tiles * splits >= BIG_MIN_TILES && big_tiles < 2147483647L && K % BK == 0) {
+  if (big_tiles * splits >= big_min_tiles() && big_tiles < 2147483647L && K % BK == 0) {
     static bool big_configured = false;
     if (!big_configured) {
       hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_mfma_big_kernel<EPI>),

@@ -29,12 +29,13 @@ from .workspace import GEMM_PART_FLOATS, KernelWorkspace, KeyRanges, Partials, P
 EPI_BF16, EPI_F32, EPI_ACCUM, EPI_SWIGLU = 0, 1, 2, 3
 SKINNY_MAX_ROWS = 128          # up to this many tokens the weight-streaming kernels serve a product (measured against the tile kernel)
 ROWS_PER_BLOCK = 32            # weight rows per block of the skinny kernel
-TARGET_BLOCKS = 512            # blocks wanted in flight to keep HBM busy
+BLOCKS_PER_UNIT = 2            # blocks of it wanted per compute unit to keep HBM busy (measured: 512 on 256 units; 384 and 768 are slower)
 SHARED_FROM_TOKENS = 32        # more tokens than this: the skinny kernel that shares activations per block ...
 SHARED_ROWS_PER_BLOCK = 64     # ... with this many weight rows per block ...
-SHARED_TARGET_BLOCKS = 256     # ... and this many blocks wanted (one per compute unit)
+SHARED_BLOCKS_PER_UNIT = 1     # ... and one block wanted per compute unit
 TILE_MAX_SPLITS = 4
-BIG_MIN_TILES = 192            # 256 x 256 tiles (times k pieces) from which the large-tile kernel is taken (the library's rule)
+BIG_TILES_PER_UNIT = 0.75      # 256 x 256 tiles (times k pieces) per compute unit from which the large-tile kernel is taken (the library's rule)
+DEFAULT_UNITS = 256            # compute units assumed where no device can be asked (an MI355X)
 BIG_MIN_K = 1024               # a piece of the large-tile kernel keeps at least this much of k
 BIG_SPLIT_MIN_K = 6144         # ... and k is cut for it only from this length on
 PIECES_BELOW_TILES = 200       # fewer 128 x 128 tiles than this: q, k, v of a prompt portion are left in k pieces too
@@ -42,7 +43,7 @@ TILE_HEAD_DIMS = tuple(range(16, 257, 16))         # head sizes of the prompt-at
 DECODE_HEAD_DIMS = tuple(range(16, 257, 16))       # head sizes of the key-split decode kernel
 FUSED_DECODE_HEAD_DIMS = (64, 128)                 # ... and of its form that starts from the q|k|v projection (whole halves of a head per fragment)
 MAX_DECODE_SPLITS = 64         # the combine kernel holds one key range per lane
-DECODE_WAVES_WANTED = 512      # waves of the decode attention kernel that fill the chip (measured at batch 1 to 64: more is never faster)
+DECODE_WAVES_PER_UNIT = 2      # waves of the decode attention kernel per compute unit that fill the chip (measured at batch 1 to 64: more is never faster)
 DECODE_MIN_KEYS_PER_SPLIT = 128
 
 
@@ -50,15 +51,30 @@ def _stream() -> int:
     return _lib.current_stream()
 
 
+@functools.lru_cache(maxsize=None)
+def _units_of(index: int) -> int:
+    return int(torch.cuda.get_device_properties(index).multi_processor_count)
+
+
+def compute_units() -> int:
+    """Compute units of the current device: the split rules below count blocks and waves in
+    multiples of it (256 on an MI355X, where they were measured)."""
+    try:
+        return _units_of(torch.cuda.current_device())
+    except Exception:                    # no device in this process (rules asked for on the host)
+        return DEFAULT_UNITS
+
+
 def _gemm_ok(a, w, K, lda, ldw) -> bool:
     return K % 8 == 0 and lda % 8 == 0 and ldw % 8 == 0 and a.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
 
 
 def _skinny_splits(M: int, N: int, K: int) -> int:
+    units = compute_units()
     if M > SHARED_FROM_TOKENS:     # the kernel that shares an activation tile per block: one block per compute unit
-        groups, wanted = -(-N // SHARED_ROWS_PER_BLOCK), SHARED_TARGET_BLOCKS
+        groups, wanted = -(-N // SHARED_ROWS_PER_BLOCK), SHARED_BLOCKS_PER_UNIT * units
     else:
-        groups, wanted = -(-N // ROWS_PER_BLOCK), TARGET_BLOCKS
+        groups, wanted = -(-N // ROWS_PER_BLOCK), BLOCKS_PER_UNIT * units
     splits = max(1, min(-(-wanted // groups), K // 256))
     while splits > 1 and splits * M * N > GEMM_PART_FLOATS:
         splits -= 1
@@ -68,6 +84,7 @@ def _skinny_splits(M: int, N: int, K: int) -> int:
 def _tile_splits(M: int, N: int, K: int) -> int:
     """k-split of the tile kernels: only when the output has too few tiles to fill the chip."""
     big = -(-M // 256) * -(-N // 256)
+    units = compute_units()
     if K % 64 == 0:
         # a long k over few 256 x 256 tiles (the down projection of a 2,048-token prompt): as many
         # pieces on the large-tile kernel as give every compute unit one block (measured at
@@ -77,11 +94,11 @@ def _tile_splits(M: int, N: int, K: int) -> int:
         # o projection of such a prompt (k = 3,072 / 4,096, two pieces) took 68 / 93 us with its
         # norm against 61 / 86 us unsplit on the small tiles
         for pieces in (4, 3, 2):
-            if (BIG_MIN_TILES <= big * pieces <= 256 and K >= max(pieces * BIG_MIN_K, BIG_SPLIT_MIN_K)
+            if (BIG_TILES_PER_UNIT * units <= big * pieces <= units and K >= max(pieces * BIG_MIN_K, BIG_SPLIT_MIN_K)
                     and pieces * M * N <= GEMM_PART_FLOATS):
                 return pieces
     tiles = -(-M // 128) * -(-N // 128)
-    splits = min(TILE_MAX_SPLITS, TARGET_BLOCKS // max(1, tiles), K // 512)
+    splits = min(TILE_MAX_SPLITS, BLOCKS_PER_UNIT * units // max(1, tiles), K // 512)
     while splits > 1 and splits * M * N > GEMM_PART_FLOATS:
         splits -= 1
     return max(1, splits)
@@ -465,7 +482,7 @@ def decode_length_bucket(max_kv_len: int) -> int:
 def decode_splits(R: int, num_kv_heads: int, max_kv_len: int) -> int:
     """Key ranges per (request, kv head): enough waves to fill the chip, no more than the
     keys of the step's length bucket are worth."""
-    splits = max(1, min(MAX_DECODE_SPLITS, -(-DECODE_WAVES_WANTED // (R * num_kv_heads))))
+    splits = max(1, min(MAX_DECODE_SPLITS, -(-DECODE_WAVES_PER_UNIT * compute_units() // (R * num_kv_heads))))
     return min(splits, max(1, decode_length_bucket(max_kv_len) // DECODE_MIN_KEYS_PER_SPLIT))
 
 
