@@ -214,3 +214,41 @@ def test_mixed_requests_on_a_windowed_model(toy, tmp_path, dtype):
     check(run_trace(runner, steps, str(tmp_path)), toy, reqs, dtype, "mixed")
     runner.cache.check_invariants()
     assert runner.cache.num_live == 0 and all(runner.cache.free_pages(g) == runner.num_pages for g in range(3))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_engine_with_graphs_on_a_windowed_model(toy, dtype):
+    """``ContinuousBatchEngine`` with its default options (decode steps replayed from graphs, a step
+    launched ahead) over the three cache groups: the graphs' block tables are as wide as the length
+    bucket while the windowed groups' early columns hold no page any more, contexts pass the windows
+    and several buckets, requests end at different steps.  The tokens are those of eager steps, the
+    greedy ones the plain implementation's arg max, and every page comes back."""
+    from photon_infer_amd import ContinuousBatchEngine
+    d, raw, W = toy
+    prompts = [random_tokens(n, 300, 70 + n) for n in (90, 20, 150, 45)]
+    new = [70, 140, 40, 100]                    # contexts reach 160, 160, 190, 145: past both windows and past 128
+    temps = [0.0, 0.9, 0.0, 0.7]
+
+    def run(**kw):
+        eng = ContinuousBatchEngine(d, dtype=dtype, block_size=PAGE, num_blocks=64, max_batch=4, chunk_size=64,
+                                    max_step_tokens=96, **kw)
+        ids = [eng.add_request(p, n, temperature=t, seed=5 + i, ignore_eos=True) for i, (p, n, t) in enumerate(zip(prompts, new, temps))]
+        eng.run_until_complete()
+        assert eng.runner.cache.num_live == 0 and all(eng.runner.cache.free_pages(g) == 64 for g in range(3))
+        eng.runner.cache.check_invariants()
+        return [eng.get_result(i) for i in ids], eng
+
+    eager, _ = run(use_graphs=False, lookahead=False)
+    graphed, eng = run()
+    assert eng.runner.graph_safe and len(eng.runner._graphs) >= 3 and len({b for _, b in eng.runner._graphs}) >= 2
+    assert graphed == eager
+    for p, out, t in zip(prompts, graphed, temps):
+        if t > 0:
+            continue
+        seq = list(p) + list(out)
+        ref = plain_window_toy(raw, W, seq)
+        emu = plain_window_toy(raw, W, seq, act_round=P.bf16_round) if dtype == "bfloat16" else ref
+        slack = 1e-4 if dtype == "float32" else 3.0 * (emu - ref).abs().max().item()
+        for k, tok in enumerate(out):
+            row = ref[len(p) - 1 + k]
+            assert row[tok].item() >= row.max().item() - 2 * slack, (len(p), k, tok)
