@@ -58,6 +58,17 @@ template <> __host__ __device__ inline bf16_t from_float<bf16_t>(float v) {
   return r;
 }
 
+// four consecutive elements as float32 (16-byte aligned float32, 8-byte aligned bfloat16)
+__device__ inline void load4(const float* p, float v[4]) {
+  const float4 q = *reinterpret_cast<const float4*>(p);
+  v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w;
+}
+__device__ inline void load4(const bf16_t* p, float v[4]) {
+  const uint2 q = *reinterpret_cast<const uint2*>(p);
+  v[0] = __uint_as_float(q.x << 16); v[1] = __uint_as_float(q.x & 0xffff0000u);
+  v[2] = __uint_as_float(q.y << 16); v[3] = __uint_as_float(q.y & 0xffff0000u);
+}
+
 // ---- wave64 reductions (every lane gets the result)
 __device__ inline float wave_sum(float v) {
 #pragma unroll

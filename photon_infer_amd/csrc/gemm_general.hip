@@ -8,6 +8,12 @@
 //
 // Each output element accumulates over k in ascending order, 16 at a time, so a row's
 // result does not depend on which other rows share the launch.
+//
+// Up to 16 rows of activations (decode steps) take a second kernel that streams the weights:
+// a wave owns a few weight rows, its lanes walk k four elements at a time (16-byte loads that
+// follow the row), the activations of a k chunk are shared through LDS, and every output is
+// summed over the lanes at the end.  A lane adds its own k in ascending order and the lanes are
+// added in a fixed tree, so here too a row's result does not depend on the other rows.
 #include "common.h"
 
 #define GT 64   // output tile edge
@@ -64,9 +70,92 @@ __global__ __launch_bounds__(256) void gemm_general_kernel(TC* __restrict__ C, l
   }
 }
 
+// ------------------------------------------------------------------ few rows: stream the weights
+#define ROWS_KC 512   // k per chunk of activations in LDS
+
+// MT: rows of activations the kernel holds (M <= MT); R: weight rows per wave.  K and the row
+// strides are multiples of 4 and the operands 16-byte aligned (8-byte for bfloat16).
+template <typename TA, typename TW, typename TC, bool ACCUM, int MT, int R>
+__global__ __launch_bounds__(256) void gemm_rows_kernel(TC* __restrict__ C, long ldc, const TA* __restrict__ A, long lda,
+                                                        const TW* __restrict__ W, long ldw, int M, int N, int K) {
+  static_assert(R * MT <= PI_WAVE, "one lane per output of a wave");
+  __shared__ __attribute__((aligned(16))) float As[MT][ROWS_KC];
+  const int tid = threadIdx.x, lane = tid % PI_WAVE, wave = tid / PI_WAVE;
+  const long n0 = ((long)blockIdx.x * 4 + wave) * R;
+  const TW* wrow[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) wrow[r] = W + (n0 + r < N ? n0 + r : (long)N - 1) * ldw;   // rows beyond N: the last row, never stored
+  float acc[R][MT];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) acc[r][m] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += ROWS_KC) {
+    for (int idx = tid; idx < MT * (ROWS_KC / 4); idx += 256) {
+      const int m = idx / (ROWS_KC / 4), kl = (idx % (ROWS_KC / 4)) * 4;
+      float v[4] = {0.f, 0.f, 0.f, 0.f};
+      if (m < M && k0 + kl < K) load4(A + (long)m * lda + k0 + kl, v);
+      *reinterpret_cast<float4*>(&As[m][kl]) = make_float4(v[0], v[1], v[2], v[3]);
+    }
+    __syncthreads();
+#pragma unroll
+    for (int sub = 0; sub < ROWS_KC / (4 * PI_WAVE); ++sub) {
+      const int kl = sub * 4 * PI_WAVE + lane * 4;
+      if (k0 + kl < K) {
+        float w[R][4];
+#pragma unroll
+        for (int r = 0; r < R; ++r) load4(wrow[r] + k0 + kl, w[r]);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const float4 a = *reinterpret_cast<const float4*>(&As[m][kl]);
+#pragma unroll
+          for (int r = 0; r < R; ++r) {
+            acc[r][m] = fmaf(a.x, w[r][0], acc[r][m]);
+            acc[r][m] = fmaf(a.y, w[r][1], acc[r][m]);
+            acc[r][m] = fmaf(a.z, w[r][2], acc[r][m]);
+            acc[r][m] = fmaf(a.w, w[r][3], acc[r][m]);
+          }
+        }
+      }
+    }
+    __syncthreads();
+  }
+  // every output summed over the lanes; lane r * MT + m keeps output (m, n0 + r)
+  float mine = 0.f;
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const float total = wave_sum(acc[r][m]);
+      if (lane == r * MT + m) mine = total;
+    }
+  const int r = lane / MT, m = lane % MT;
+  if (lane < R * MT && m < M && n0 + r < N) {
+    TC* c = C + (long)m * ldc + n0 + r;
+    *c = ACCUM ? from_float<TC>(to_float(*c) + mine) : from_float<TC>(mine);
+  }
+}
+
+template <typename TA, typename TW, typename TC>
+static int launch_rows(void* C, long ldc, const void* A, long lda, const void* W, long ldw, int M, int N, int K, int accumulate,
+                       hipStream_t stream) {
+  const dim3 block(256);
+#define ROWS_GO(ACC, MT, R) hipLaunchKernelGGL((gemm_rows_kernel<TA, TW, TC, ACC, MT, R>), dim3(ceil_div(N, 4 * R)), block, 0, stream, \
+                                               (TC*)C, ldc, (const TA*)A, lda, (const TW*)W, ldw, M, N, K)
+  if (M <= 8) {
+    if (accumulate) ROWS_GO(true, 8, 4); else ROWS_GO(false, 8, 4);
+  } else {
+    if (accumulate) ROWS_GO(true, 16, 2); else ROWS_GO(false, 16, 2);
+  }
+#undef ROWS_GO
+  return pi_check_launch("gemm_rows");
+}
+
 template <typename TA, typename TW, typename TC>
 static int launch(void* C, long ldc, const void* A, long lda, const void* W, long ldw, int M, int N, int K, int accumulate,
                   hipStream_t stream) {
+  if (M <= 16 && K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0 && (long)ceil_div(N, 8) < 2147483647L)
+    return launch_rows<TA, TW, TC>(C, ldc, A, lda, W, ldw, M, N, K, accumulate, stream);
   const dim3 grid(ceil_div(N, GT), ceil_div(M, GT)), block(256);
   if (grid.y > 65535) return pi_fail("gemm: too many rows (%d)", M);
   if (accumulate)

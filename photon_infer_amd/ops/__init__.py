@@ -403,10 +403,20 @@ def paged_attention(out: torch.Tensor, q: torch.Tensor, k_cache: torch.Tensor, v
         if fast.paged_attention(out, q, k_cache, v_cache, block_table, ctx, num_heads, num_kv_heads, head_dim,
                                 page_size, scale, window, pages, ws):
             return
+    # a step of few tokens over long contexts: its keys cut into ranges, merged by a second kernel
+    # (as many as the context-length bucket asks for, so that a step gives the same bits eagerly and replayed)
+    ranges = general_attention_ranges(T, num_heads, int(ctx.max_kv_len))
+    part = torch.empty(T * num_heads * ranges * (head_dim + 2), dtype=torch.float32, device=q.device) if ranges > 1 else None
     _lib.call("core", "pi_paged_attention_general", out.data_ptr(), _rows(out, "attention out"), q.data_ptr(),
               _rows(q, "q"), k_cache.data_ptr(), v_cache.data_ptr(), _dt(q), block_table.data_ptr(),
               block_table.shape[1], ctx.req_of_token.data_ptr(), ctx.positions.data_ptr(), T, num_heads,
-              num_kv_heads, head_dim, page_size, float(scale), int(window), pages, _stream())
+              num_kv_heads, head_dim, page_size, float(scale), int(window), pages, ranges, _ptr(part),
+              0 if part is None else part.numel(), _stream())
+
+
+def general_attention_ranges(tokens: int, num_heads: int, max_kv_len: int) -> int:
+    """Key ranges per (token, head) that the general attention kernel makes for such a step."""
+    return int(_lib.load("core").pi_paged_attention_general_ranges(tokens, num_heads, decode_length_bucket(max_kv_len)))
 
 
 def sample(out: torch.Tensor, logits: torch.Tensor, temperature: Optional[torch.Tensor] = None,

@@ -20,7 +20,8 @@ _SIGNATURES = {
         "pi_swiglu": [P, P, I, I, I, I, P],
         "pi_rope_kv_write": [P, L, P, L, P, L, I, P, P, P, I, I, I, I, I, I, I, P, P, P, I, I, L, P, I, I, I, I, I, P],
         "pi_gemm_general": [P, I, L, P, I, L, P, I, L, I, I, I, I, P],
-        "pi_paged_attention_general": [P, L, P, L, P, P, I, P, I, P, P, I, I, I, I, I, F, I, L, P],
+        "pi_paged_attention_general": [P, L, P, L, P, P, I, P, I, P, P, I, I, I, I, I, F, I, L, I, P, L, P],
+        "pi_paged_attention_general_ranges": [I, I, I],
         "pi_rope_table": [P, P, P, I, I, P],
         "pi_sample": [P, P, L, P, P, I, I, P, L, P],
         "pi_sample_static": [P, P, L, P, P, I, I, P],
