@@ -83,16 +83,37 @@ __global__ __launch_bounds__(PI_WAVE) void paged_attention_general_kernel(
     for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) acc[i] *= corr;
     __syncthreads();
     const int nk = (p - k0 + 1) < PI_WAVE ? (p - k0 + 1) : PI_WAVE;
-    for (int kk = 0; kk < nk; ++kk) {
+    // keys in ascending order; four at a time where they lie side by side in a page (values are
+    // stored with the slot as the last axis), in the same order of additions
+    for (int kk = 0; kk < nk;) {
       const long o2 = voff[kk];
-      if (o2 < 0) continue;
-      const T* vr = v_cache + o2;
-      const float pk = ps[kk];
+      const bool four = page_size % 4 == 0 && ((k0 + kk) & 3) == 0 && kk + 3 < nk;
+      if (o2 >= 0) {
+        const T* vr = v_cache + o2;
+        if (four) {
+          const float p0 = ps[kk], p1 = ps[kk + 1], p2 = ps[kk + 2], p3 = ps[kk + 3];
 #pragma unroll
-      for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
-        const int d = lane + i * PI_WAVE;
-        if (d < hd) acc[i] = fmaf(pk, to_float(vr[(long)d * page_size]), acc[i]);
+          for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
+            const int d = lane + i * PI_WAVE;
+            if (d < hd) {
+              float vv[4];
+              load4(vr + (long)d * page_size, vv);
+              acc[i] = fmaf(p0, vv[0], acc[i]);
+              acc[i] = fmaf(p1, vv[1], acc[i]);
+              acc[i] = fmaf(p2, vv[2], acc[i]);
+              acc[i] = fmaf(p3, vv[3], acc[i]);
+            }
+          }
+        } else {
+          const float pk = ps[kk];
+#pragma unroll
+          for (int i = 0; i < PI_MAX_HEAD_DIM / PI_WAVE; ++i) {
+            const int d = lane + i * PI_WAVE;
+            if (d < hd) acc[i] = fmaf(pk, to_float(vr[(long)d * page_size]), acc[i]);
+          }
+        }
       }
+      kk += four ? 4 : 1;
     }
     m = m_new;
     __syncthreads();
