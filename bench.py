@@ -11,7 +11,8 @@ own path, driven as the engine drives its decode phase: metadata upload, the rep
 (model + sampling kernel) that takes its tokens from the step before it on the device, and
 the copy of the chosen tokens to the host, which reads every step's tokens one step late.
 Also on the line: ``prefill`` (one 2,048-token prompt in one step), ``roofline`` (bytes the
-decode step has to read / its time, against 8 TB/s) and ``points`` (batch 1 and 64).
+decode step has to read / its time, against 8 TB/s) and ``points`` (batch 1 and 64, and
+``decode_b8_fp32``: the headline's decode step on the float32 path).
 ``points`` also holds ``engine_b8``: decoded tokens per second of the same batch through
 ``ContinuousBatchEngine`` (scheduler, request objects, sampling, the step ahead), measured over its
 decode phase.
@@ -528,6 +529,15 @@ def main() -> int:
         if not synthetic:
             points[f"engine_b{args.batch}"] = round(
                 args.batch / time_engine_decode(runner, args.batch, args.steps, args.warmup, context), 1)
+        if args.dtype == "bf16":
+            # the same decode step on the float32 path (true 32-bit kernels, caches of random numbers)
+            import gc
+            del runner
+            gc.collect()
+            torch.cuda.empty_cache()
+            runner32, _ = make_runner(MODEL, args.layers, "fp32", args.batch, args.batch * (context + 64), max_model_len=context + 64)
+            s32, _ = time_decode(runner32, args.batch, min(args.steps, 16), min(args.warmup, 2), context, synthetic_cache=True)
+            points[f"decode_b{args.batch}_fp32"] = round(args.batch / s32, 1)
         line["points"] = points
     print(json.dumps(line), flush=True)
     return 0

@@ -180,3 +180,52 @@ def test_two_layers_at_the_benchmark_sizes_against_the_plain_implementation(monk
         err = max((g - r).abs().max().item() for g, r in zip(got[i], ref))
         assert err <= tol, (i, len(p), err, tol)
         assert tol < 0.2 * ref.abs().max().item()             # the yardstick itself is tight
+
+
+def test_float32_decoding_over_key_ranges_equals_the_plain_implementation(model_dirs):
+    """The float32 path at contexts where its attention kernel cuts a decoding token's keys into
+    ranges (from 256 keys on) and its products take the weight-streaming kernel for few rows:
+    single tokens through ``step`` and through ``decode_step`` (a replayed graph) give the same
+    logits bit for bit, and they are the plain implementation's."""
+    from photon_infer_amd import ops
+    from photon_infer_amd.engine import EngineOptions, ModelRunner, StepEntry
+    cfg, W = P.read_model_folder(model_dirs["D"])
+    vocab = ALL["D"][0]["vocab_size"]
+    prompts = [random_tokens(n, vocab, 700 + n) for n in (300, 530, 40)]
+    steps = 24
+    assert ops.general_attention_ranges(3, ALL["D"][0]["num_attention_heads"], 531) > 1
+
+    def run(graphs):
+        runner = ModelRunner(model_dirs["D"], EngineOptions(dtype="float32", block_size=16, num_blocks=96, max_batch=3,
+                                                            use_graphs=graphs, keep_logits=True))
+        seqs, rows = [list(p) for p in prompts], [[] for _ in prompts]
+        for i, p in enumerate(prompts):
+            runner.admit(i)
+            logits = runner.step([StepEntry(i, p, [len(p) - 1])])
+            rows[i].append(logits[0].cpu())
+            seqs[i].append(int(logits[0].argmax()))
+        for _ in range(steps):
+            entries = [StepEntry(i, [s[-1]], [0]) for i, s in enumerate(seqs)]
+            if graphs:
+                ids = runner.decode_step(entries, [0.0] * 3, [0.0] * 3).tolist()
+                logits = runner.decode_logits.cpu()
+            else:
+                logits = runner.step(entries).cpu()
+                ids = [int(r.argmax()) for r in logits]
+            for i, tok in enumerate(ids):
+                rows[i].append(logits[i].clone())
+                seqs[i].append(tok)
+        assert bool(runner._graphs) == graphs
+        return seqs, rows
+
+    seqs, eager = run(False)
+    seqs_g, graphed = run(True)
+    assert seqs_g == seqs
+    for a, b in zip(eager, graphed):
+        assert all(torch.equal(x, y) for x, y in zip(a, b))           # the same bits, eagerly and replayed
+    for i, p in enumerate(prompts):
+        seq = seqs[i][:-1]
+        ref = PW.llama_forward(cfg, W, seq, list(range(len(p) - 1, len(seq))), device="cuda").cpu()
+        tol = 3e-5 * max(1.0, ref.abs().max().item())
+        err = max((g - r).abs().max().item() for g, r in zip(eager[i], ref))
+        assert err <= tol, (i, err, tol)
