@@ -10,10 +10,11 @@
 // result does not depend on which other rows share the launch.
 //
 // Up to 16 rows of activations (decode steps) take a second kernel that streams the weights:
-// a wave owns a few weight rows, its lanes walk k four elements at a time (16-byte loads that
+// a block owns a few weight rows, its waves take turns over k, their lanes four elements at a time (16-byte loads that
 // follow the row), the activations of a k chunk are shared through LDS, and every output is
-// summed over the lanes at the end.  A lane adds its own k in ascending order and the lanes are
-// added in a fixed tree, so here too a row's result does not depend on the other rows.
+// summed over the lanes and waves at the end.  A lane adds its own k in ascending order and the
+// lanes and waves are added in a fixed order, so here too a row's result does not depend on the
+// other rows.
 #include "common.h"
 
 #define GT 64   // output tile edge
@@ -71,17 +72,23 @@ __global__ __launch_bounds__(256) void gemm_general_kernel(TC* __restrict__ C, l
 }
 
 // ------------------------------------------------------------------ few rows: stream the weights
-#define ROWS_KC 512   // k per chunk of activations in LDS
 
-// MT: rows of activations the kernel holds (M <= MT); R: weight rows per wave.  K and the row
+// MT: rows of activations the kernel holds (M <= MT); R: weight rows per wave.  KW = 1: a block's
+// four waves take R rows each; KW = 4: they work on the same R rows, each on every fourth group
+// of 256 k, and their sums meet in LDS and are added in wave order (matrices of few rows, which
+// would otherwise leave most of the chip idle, and steps of one or two tokens).  K and the row
 // strides are multiples of 4 and the operands 16-byte aligned (8-byte for bfloat16).
-template <typename TA, typename TW, typename TC, bool ACCUM, int MT, int R>
+template <typename TA, typename TW, typename TC, bool ACCUM, int MT, int R, int KW>
 __global__ __launch_bounds__(256) void gemm_rows_kernel(TC* __restrict__ C, long ldc, const TA* __restrict__ A, long lda,
                                                         const TW* __restrict__ W, long ldw, int M, int N, int K) {
   static_assert(R * MT <= PI_WAVE, "one lane per output of a wave");
+  static_assert(KW == 1 || KW == 4, "the waves of a block share their rows or do not");
+  constexpr int ROWS_KC = (8192 / MT) < 1024 ? 1024 : (8192 / MT) > 4096 ? 4096 : (8192 / MT);   // k per chunk of activations in LDS
+  constexpr int GROUP = 4 * PI_WAVE;             // k a wave covers with one load per lane and row
   __shared__ __attribute__((aligned(16))) float As[MT][ROWS_KC];
+  __shared__ float sums[4][R * MT];
   const int tid = threadIdx.x, lane = tid % PI_WAVE, wave = tid / PI_WAVE;
-  const long n0 = ((long)blockIdx.x * 4 + wave) * R;
+  const long n0 = KW == 1 ? ((long)blockIdx.x * 4 + wave) * R : (long)blockIdx.x * R;
   const TW* wrow[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) wrow[r] = W + (n0 + r < N ? n0 + r : (long)N - 1) * ldw;   // rows beyond N: the last row, never stored
@@ -99,8 +106,8 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(TC* __restrict__ C, long
     }
     __syncthreads();
 #pragma unroll
-    for (int sub = 0; sub < ROWS_KC / (4 * PI_WAVE); ++sub) {
-      const int kl = sub * 4 * PI_WAVE + lane * 4;
+    for (int sub = 0; sub < ROWS_KC / GROUP / KW; ++sub) {
+      const int kl = (KW == 1 ? sub : sub * 4 + wave) * GROUP + lane * 4;      // this wave's group of the chunk
       if (k0 + kl < K) {
         float w[R][4];
 #pragma unroll
@@ -120,7 +127,8 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(TC* __restrict__ C, long
     }
     __syncthreads();
   }
-  // every output summed over the lanes; lane r * MT + m keeps output (m, n0 + r)
+  // every output summed over the lanes of its wave (then over the waves, in wave order); lane
+  // (or thread) r * MT + m keeps output (m, n0 + r)
   float mine = 0.f;
 #pragma unroll
   for (int r = 0; r < R; ++r)
@@ -129,6 +137,12 @@ __global__ __launch_bounds__(256) void gemm_rows_kernel(TC* __restrict__ C, long
       const float total = wave_sum(acc[r][m]);
       if (lane == r * MT + m) mine = total;
     }
+  if (KW == 4) {
+    if (lane < R * MT) sums[wave][lane] = mine;
+    __syncthreads();
+    if (wave != 0) return;
+    if (lane < R * MT) mine = ((sums[0][lane] + sums[1][lane]) + sums[2][lane]) + sums[3][lane];
+  }
   const int r = lane / MT, m = lane % MT;
   if (lane < R * MT && m < M && n0 + r < N) {
     TC* c = C + (long)m * ldc + n0 + r;
@@ -140,13 +154,24 @@ template <typename TA, typename TW, typename TC>
 static int launch_rows(void* C, long ldc, const void* A, long lda, const void* W, long ldw, int M, int N, int K, int accumulate,
                        hipStream_t stream) {
   const dim3 block(256);
-#define ROWS_GO(ACC, MT, R) hipLaunchKernelGGL((gemm_rows_kernel<TA, TW, TC, ACC, MT, R>), dim3(ceil_div(N, 4 * R)), block, 0, stream, \
-                                               (TC*)C, ldc, (const TA*)A, lda, (const TW*)W, ldw, M, N, K)
-  if (M <= 8) {
-    if (accumulate) ROWS_GO(true, 8, 4); else ROWS_GO(false, 8, 4);
+#define ROWS_GO(ACC, MT, R, KW) hipLaunchKernelGGL((gemm_rows_kernel<TA, TW, TC, ACC, MT, R, KW>), dim3(ceil_div(N, R * (KW == 1 ? 4 : 1))), block, 0, \
+                                                   stream, (TC*)C, ldc, (const TA*)A, lda, (const TW*)W, ldw, M, N, K)
+#define ROWS_PICK(MT, R1, R4)                                                                    \
+  do {                                                                                           \
+    if (few_rows) { if (accumulate) ROWS_GO(true, MT, R4, 4); else ROWS_GO(false, MT, R4, 4); }  \
+    else { if (accumulate) ROWS_GO(true, MT, R1, 1); else ROWS_GO(false, MT, R1, 1); }           \
+  } while (0)
+  // a matrix of few rows gives too few blocks when every wave takes rows of its own: its blocks'
+  // waves share their rows and split k instead
+  const bool few_rows = N < 8192;
+  if (M <= 2) {
+    if (accumulate) ROWS_GO(true, 2, 8, 4); else ROWS_GO(false, 2, 8, 4);
+  } else if (M <= 8) {
+    ROWS_PICK(8, 4, 8);
   } else {
-    if (accumulate) ROWS_GO(true, 16, 2); else ROWS_GO(false, 16, 2);
+    ROWS_PICK(16, 2, 4);
   }
+#undef ROWS_PICK
 #undef ROWS_GO
   return pi_check_launch("gemm_rows");
 }
@@ -154,7 +179,7 @@ static int launch_rows(void* C, long ldc, const void* A, long lda, const void* W
 template <typename TA, typename TW, typename TC>
 static int launch(void* C, long ldc, const void* A, long lda, const void* W, long ldw, int M, int N, int K, int accumulate,
                   hipStream_t stream) {
-  if (M <= 16 && K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0 && (long)ceil_div(N, 8) < 2147483647L)
+  if (M <= 16 && K % 4 == 0 && lda % 4 == 0 && ldw % 4 == 0 && (uintptr_t)A % 16 == 0 && (uintptr_t)W % 16 == 0 && (long)N < 2147483647L)
     return launch_rows<TA, TW, TC>(C, ldc, A, lda, W, ldw, M, N, K, accumulate, stream);
   const dim3 grid(ceil_div(N, GT), ceil_div(M, GT)), block(256);
   if (grid.y > 65535) return pi_fail("gemm: too many rows (%d)", M);
