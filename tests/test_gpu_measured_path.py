@@ -179,18 +179,29 @@ def test_two_layers_at_the_benchmark_sizes_against_the_plain_implementation(monk
         assert (8, 2048, 2048, 8) in calls["skinny"] and (8, 2048, 8192, 8) in calls["skinny"], set(calls["skinny"])
     elif size == "8b":
         assert counts["ranges_merged_by_product"] == 0        # its o matrix (32 MB) is streamed by the plain kernel, the ranges merged before
+    # one mixed step on top: a 300-token portion for the request that is 146 tokens long, a
+    # 40-token one for the longest, single tokens for the rest (the tile kernel and the key-split
+    # kernel share the step; the portions' products take the tile kernels, fed late in a context)
+    more = {4: random_tokens(300, cfg.vocab_size, 901), 0: random_tokens(40, cfg.vocab_size, 902)}
+    entries, fed = [], []
+    for i, rid in enumerate(rids):
+        toks = [seqs[i][-1]] + more[i] if i in more else [seqs[i][-1]]
+        entries.append(StepEntry(rid, toks, [len(toks) - 1]))
+        fed.append(toks)
+    mixed = runner.step(entries).cpu()
     for rid in rids:
         runner.release(rid)
+    assert runner.cache.free_pages() == runner.num_pages
 
     raw = cfg.to_dict()
     for i, p in enumerate(prompts):
-        seq = seqs[i][:-1]                                    # the last token was chosen and never fed
-        rows = list(range(len(p) - 1, len(seq)))
-        assert len(rows) == steps + 1 == len(got[i])
+        seq = seqs[i][:-1] + fed[i]                           # everything that was fed
+        rows = list(range(len(p) - 1, len(seqs[i]) - 1)) + [len(seq) - 1]
+        assert len(rows) == steps + 2 == len(got[i]) + 1
         ref = PW.llama_forward(raw, plain_weights, seq, rows, device="cuda").cpu()
         emu = PW.llama_forward(raw, plain_weights, seq, rows, act_round=P.bf16_round, device="cuda").cpu()
         tol = 3.0 * (emu - ref).abs().max().item()
-        err = max((g - r).abs().max().item() for g, r in zip(got[i], ref))
+        err = max((g - r).abs().max().item() for g, r in zip(got[i] + [mixed[i]], ref))
         assert err <= tol, (i, len(p), err, tol)
         assert tol < 0.2 * ref.abs().max().item()             # the yardstick itself is tight
 
