@@ -113,6 +113,8 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(int* __restrict_
 // sum (chunk sums rescaled to the global maximum); the chunk the draw falls into; and scans that
 // chunk for the first index whose cumulative weight reaches the draw.
 #define CHUNK_REC 4   // max, index (as float bits), sum, unused
+#define TWO_STAGE_FROM 16384
+#define MAX_CHUNKS 64
 
 __global__ __launch_bounds__(SAMPLE_THREADS) void sample_stage1_kernel(float* __restrict__ ws, const float* __restrict__ logits,
                                                                        long row_stride, const float* __restrict__ temperature,
@@ -160,8 +162,12 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_stage2_kernel(int* __re
   const int row = blockIdx.x, tid = threadIdx.x;
   const float* l = logits + (long)row * row_stride;
   const float* rec = ws + (long)row * chunks * CHUNK_REC;
-  ArgMax best = {-INFINITY, 0x7fffffff};
-  for (int c = 0; c < chunks; ++c) best = better(best, ArgMax{rec[c * CHUNK_REC], __float_as_int(rec[c * CHUNK_REC + 1])});
+  // the chunks' maxima, one per lane (there are at most as many chunks as a wave has lanes): every
+  // wave finds the same overall maximum, lowest index among equals, in one trip to memory
+  static_assert(MAX_CHUNKS <= PI_WAVE, "one chunk record per lane");
+  const int lane = tid % PI_WAVE;
+  ArgMax best = lane < chunks ? ArgMax{rec[lane * CHUNK_REC], __float_as_int(rec[lane * CHUNK_REC + 1])} : ArgMax{-INFINITY, 0x7fffffff};
+  best = wave_argmax(best);
   if (best.i == 0x7fffffff) best = {l[0], 0};
   const float tau = temperature ? temperature[row] : 0.f;
   if (!(tau > 0.f)) {
@@ -230,9 +236,6 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_stage2_kernel(int* __re
 
 // Rows of more than `two_stage_from` logits use the two-stage kernels and need `ws`
 // (float32, M * chunks * 4 with chunks = pi_sample_chunks(V)).
-#define TWO_STAGE_FROM 16384
-#define MAX_CHUNKS 64
-
 extern "C" int pi_sample_chunks(int V) {
   if (V <= TWO_STAGE_FROM) return 0;
   int chunks = (V + 2047) / 2048;
