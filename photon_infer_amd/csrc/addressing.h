@@ -119,4 +119,26 @@ PI_ADDR unsigned big_lane_offset(int row, int rows, long ld, int piece) {
 }
 PI_ADDR int big_slab_bytes(int s, int slabs) { return imin(s, slabs - 1) * 64 * 2; }   // past the last slab: read it again, unused
 
+// ---------------------------------------------------------------- attention over the paged cache
+// Keys [pages, kv_heads, page, HD], values transposed [pages, kv_heads, HD, page], bfloat16.  A
+// chunk is two tiles of 16 keys; a tile lies in one page (pages hold a multiple of 16 tokens) at
+// slot .. slot + 15.  A tile whose page is missing (or whose id is no page of the pool) is read
+// from page 0 instead and counts as zero.  Bases in elements, a lane's part in bytes.
+PI_ADDR long kv_page_elems(int nkv, int page_size, int hd) { return (long)nkv * page_size * hd; }
+PI_ADDR bool kv_page_there(long page, long num_pages) { return page >= 0 && page < num_pages; }
+PI_ADDR long kv_page_or_first(long page, long num_pages) { return kv_page_there(page, num_pages) ? page : 0; }
+PI_ADDR long kv_key_tile(long page, long page_elems, int g, int page_size, int slot, int hd) {
+  return page * page_elems + (long)(g * page_size + slot) * hd;
+}
+PI_ADDR long kv_value_tile(long page, long page_elems, int g, int page_size, int slot, int hd) {
+  return page * page_elems + (long)g * page_size * hd + slot;
+}
+// key row lane % 16 of the tile, features (lane / 16) * 8 .. + 7 of a fragment of 32 (fragment ks lies ks * 64 bytes on)
+PI_ADDR unsigned kv_key_lane(int lane, int hd) { return (unsigned)((lane % 16) * hd + (lane / 16) * 8) * 2u; }
+// what a lane without features of its own reads (a head of 16, 48, .. features: the last fragment is half empty)
+PI_ADDR unsigned kv_key_lane_first(int lane, int hd) { return (unsigned)((lane % 16) * hd) * 2u; }
+PI_ADDR bool kv_lane_holds(int hd, int ks, int lane) { return ks * 32 + (lane / 16) * 8 < hd; }
+// value row db * 16 + lane % 16, keys (lane / 16) * 4 .. + 3 of the tile (8 bytes)
+PI_ADDR unsigned kv_value_lane(int lane, int db, int page_size) { return (unsigned)((db * 16 + lane % 16) * page_size + (lane / 16) * 4) * 2u; }
+
 }  // namespace addressing

@@ -21,6 +21,7 @@
 // The keys and values of a chunk are loaded into registers by attn_load and consumed by
 // attn_compute, so a caller can have the next chunk's loads in flight while it computes.
 #pragma once
+#include "addressing.h"
 #include "mfma.h"
 
 #define PI_LOG2E 1.4426950408889634f
@@ -31,7 +32,7 @@
 template <int HD>
 struct HeadFrags {
   static constexpr int KS = (HD + 31) / 32;
-  __device__ static inline bool holds(int ks, int lane) { return ks * 32 + (lane / 16) * 8 < HD; }   // false only in a half fragment
+  __device__ static inline bool holds(int ks, int lane) { return addressing::kv_lane_holds(HD, ks, lane); }   // false only in a half fragment
 };
 
 template <int HD, int CB>
@@ -145,12 +146,11 @@ struct KVLaneOffsets {
   bool tail;               // the lane holds features of the last fragment (always, unless HD % 32 == 16)
   uint32_t v[HD / 16];     // value row db * 16 + lane % 16, keys (lane / 16) * 4 ..
   __device__ inline void set(int page_size, int lane) {
-    const int lr = lane % 16, lg = lane / 16;
-    k = (uint32_t)(lr * HD + lg * 8) * 2u;
-    k0 = (uint32_t)(lr * HD) * 2u;
+    k = addressing::kv_key_lane(lane, HD);
+    k0 = addressing::kv_key_lane_first(lane, HD);
     tail = HeadFrags<HD>::holds(HeadFrags<HD>::KS - 1, lane);
 #pragma unroll
-    for (int db = 0; db < HD / 16; ++db) v[db] = (uint32_t)((db * 16 + lr) * page_size + lg * 4) * 2u;
+    for (int db = 0; db < HD / 16; ++db) v[db] = addressing::kv_value_lane(lane, db, page_size);
   }
 };
 
@@ -162,13 +162,13 @@ template <int HD>
 __device__ inline void attn_load(KVChunk<HD>& kv, const ChunkPages& cp, const bf16_t* __restrict__ k_cache,
                                  const bf16_t* __restrict__ v_cache, const KVLaneOffsets<HD>& off, int nkv, int g,
                                  int page_size, int num_pages) {
-  const long page_elems = (long)nkv * page_size * HD;
+  const long page_elems = addressing::kv_page_elems(nkv, page_size, HD);
 #pragma unroll
   for (int t = 0; t < 2; ++t) {
-    kv.have[t] = cp.page[t] >= 0 && cp.page[t] < num_pages;
-    const long pg = kv.have[t] ? cp.page[t] : 0;
-    const char* kp = reinterpret_cast<const char*>(k_cache + pg * page_elems + (long)(g * page_size + cp.slot[t]) * HD);
-    const char* vp = reinterpret_cast<const char*>(v_cache + pg * page_elems + (long)g * page_size * HD + cp.slot[t]);
+    kv.have[t] = addressing::kv_page_there(cp.page[t], num_pages);
+    const long pg = addressing::kv_page_or_first(cp.page[t], num_pages);
+    const char* kp = reinterpret_cast<const char*>(k_cache + addressing::kv_key_tile(pg, page_elems, g, page_size, cp.slot[t], HD));
+    const char* vp = reinterpret_cast<const char*>(v_cache + addressing::kv_value_tile(pg, page_elems, g, page_size, cp.slot[t], HD));
 #pragma unroll
     for (int ks = 0; ks < HeadFrags<HD>::KS; ++ks) {
       // a half fragment's upper lanes read their row's first features again and count as zero

@@ -5,7 +5,8 @@
 //
 // Walks the built-in sweep of shapes (and any given as arguments) through the lanes, waves,
 // blocks and steps of gemm_skinny_kernel, gemm_skinny_shared_kernel, gemm_mfma_kernel and
-// gemm_mfma_big_kernel exactly as the kernels walk them, with the matrices row by row (two row
+// gemm_mfma_big_kernel exactly as the kernels walk them (and, in the built-in sweep, through the
+// key and value fetches of the attention kernels' chunks for every head size and several page sizes), with the matrices row by row (two row
 // strides) and, where the sizes allow, in the weight-streaming kernels' tiled order.  Prints
 // "ok <fetches>" or the first fetch that leaves its operand (exit status 1).
 // "only" leaves the built-in sweep out.  "old-standin" replaces the stand-in address of a lane beyond a partial k step by the formula
@@ -171,6 +172,57 @@ static bool tiles(const Shape& s, long lda, long ldw, bool big) {
   return true;
 }
 
+// ------------------------------------------------------------------ attention over the paged cache
+// Every fetch of a chunk's two tiles (attn_load): the keys' fragments (16 bytes) and the values'
+// (8 bytes) of every lane, for a page that is there, one that is missing and one whose id is no
+// page of the pool (both read page 0 instead), lie inside the (page, kv head) block of their pool.
+static bool attention(int hd, int page_size, int nkv, long num_pages) {
+  const long page_elems = A::kv_page_elems(nkv, page_size, hd);
+  const long pool_bytes = num_pages * page_elems * 2;
+  const int KS = (hd + 31) / 32;
+  const long ids[] = {0, num_pages - 1, -1, num_pages, num_pages + 5};
+  for (long id : ids)
+    for (int g = 0; g < nkv; ++g)
+      for (int slot = 0; slot + 16 <= page_size; slot += 16) {
+        const long pg = A::kv_page_or_first(id, num_pages);
+        if (A::kv_page_there(id, num_pages) != (id >= 0 && id < num_pages) || pg < 0 || pg >= num_pages) {
+          std::printf("out of bounds: attention page id %ld of %ld pages becomes %ld\n", id, num_pages, pg);
+          return false;
+        }
+        const long block0 = ((pg * nkv + g) * (long)page_size) * hd * 2, block1 = block0 + (long)page_size * hd * 2;   // bytes of this (page, kv head)
+        for (int lane = 0; lane < 64; ++lane) {
+          for (int ks = 0; ks < KS; ++ks) {
+            const bool held = hd % 32 == 0 || ks + 1 < KS || A::kv_lane_holds(hd, KS - 1, lane);
+            const long at = A::kv_key_tile(pg, page_elems, g, page_size, slot, hd) * 2 + (held ? A::kv_key_lane(lane, hd) + ks * 64 : A::kv_key_lane_first(lane, hd));
+            ++fetches;
+            if (at < block0 || at + 16 > block1 || at + 16 > pool_bytes) {
+              std::printf("out of bounds: attention key fetch hd=%d page=%d kv heads=%d g=%d slot=%d lane=%d ks=%d at %ld\n", hd, page_size, nkv, g, slot, lane, ks, at);
+              return false;
+            }
+            const long row = (at - block0) / (hd * 2);        // the key it belongs to: one of the tile's sixteen
+            if (row != slot + lane % 16) {
+              std::printf("out of bounds: attention key fetch of lane %d reads key %ld of the page, not %d\n", lane, row, slot + lane % 16);
+              return false;
+            }
+          }
+          for (int db = 0; db < hd / 16; ++db) {
+            const long at = A::kv_value_tile(pg, page_elems, g, page_size, slot, hd) * 2 + A::kv_value_lane(lane, db, page_size);
+            ++fetches;
+            if (at < block0 || at + 8 > block1) {
+              std::printf("out of bounds: attention value fetch hd=%d page=%d kv heads=%d g=%d slot=%d lane=%d db=%d at %ld\n", hd, page_size, nkv, g, slot, lane, db, at);
+              return false;
+            }
+            const long col = ((at - block0) / 2) % page_size;  // its first key: four of the tile's sixteen per lane group
+            if (col != slot + (lane / 16) * 4) {
+              std::printf("out of bounds: attention value fetch of lane %d starts at key %ld, not %d\n", lane, col, slot + (lane / 16) * 4);
+              return false;
+            }
+          }
+        }
+      }
+  return true;
+}
+
 static bool check(const Shape& s) {
   for (int pad = 0; pad <= 16; pad += 8) {             // row strides K, K + 8, K + 16
     const long ld = s.K + pad;
@@ -209,6 +261,11 @@ int main(int argc, char** argv) {
           if (S == 1 || K / S >= 8) shapes.push_back(Shape{M, N, K, S});
   for (const Shape& s : shapes)
     if (!check(s)) return 1;
+  if (sweep)
+    for (int hd = 16; hd <= 256; hd += 16)
+      for (int page_size : {16, 32, 48, 64})
+        for (int nkv : {1, 3, 8})
+          if (!attention(hd, page_size, nkv, 7)) return 1;
   std::printf("ok %ld\n", fetches);
   return 0;
 }

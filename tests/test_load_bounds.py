@@ -5,7 +5,9 @@ value, so no comparison of results can see where it went; it faults only when th
 where its mapping ends.  The kernels take their address arithmetic from ``csrc/addressing.h``;
 ``tests/cpp/load_bounds.cpp`` includes the same header, walks every block, wave, lane and step of
 the weight-streaming kernels (row-major and tiled weights) and of the two tile kernels (their
-buffer descriptors and lane offsets) for a sweep of shapes, and checks every fetch.
+buffer descriptors and lane offsets) for a sweep of shapes, and the key and value fetches of the
+attention kernels' chunks (pages that are there, missing, or no pages of the pool) for every head
+size, and checks every fetch.
 """
 import os
 import subprocess
