@@ -252,3 +252,18 @@ def test_the_decision_to_copy_the_weights_for_streaming():
     with pytest.raises(OutOfMemoryError, match="stream_copies=True") as err:
         stream_copies_wanted(150 * GiB, 140 * GiB, asked=True)
     assert err.value.code == ErrorCode.OUT_OF_MEMORY
+
+
+def test_kernels_launch_on_the_current_devices_stream(monkeypatch):
+    """The stream handle that every kernel launch takes is asked for anew each time, for the
+    device that is current then: a process may hold runners on several devices (a runner makes
+    its own device current around its calls)."""
+    from photon_infer_amd.ops import _lib
+
+    current = {"device": 0}
+    asked = []
+    monkeypatch.setattr(_lib, "_CURRENT_DEVICE", lambda: current["device"])
+    monkeypatch.setattr(_lib, "_RAW_STREAM", lambda index: asked.append(index) or 1000 + index)
+    assert _lib.current_stream() == 1000
+    current["device"] = 3
+    assert _lib.current_stream() == 1003 and asked == [0, 3]
